@@ -32,6 +32,7 @@ class CacheError(RuntimeError):
 class GroupShape:
     num_pages: int
     window: Optional[int] = None  # None: every token is kept
+    keep_first: int = 0  # with a window: the first tokens whose pages are never given back
 
 
 _I32P = ctypes.POINTER(ctypes.c_int32)
@@ -42,7 +43,7 @@ def _bind(lib: ctypes.CDLL) -> None:
         return
     lib.ycm_last_error.restype = ctypes.c_char_p
     lib.ycm_create.restype = ctypes.c_void_p
-    lib.ycm_create.argtypes = [ctypes.c_int32, ctypes.c_int32, _I32P, _I32P, ctypes.c_int32]
+    lib.ycm_create.argtypes = [ctypes.c_int32, ctypes.c_int32, _I32P, _I32P, _I32P, ctypes.c_int32]
     lib.ycm_destroy.argtypes = [ctypes.c_void_p]
     lib.ycm_destroy.restype = None
     for name, args, res in [
@@ -78,7 +79,8 @@ class PageManager:
         n = len(self.groups)
         pages = (ctypes.c_int32 * max(n, 1))(*[g.num_pages for g in self.groups])
         wins = (ctypes.c_int32 * max(n, 1))(*[(g.window or 0) for g in self.groups])
-        self.h = self.lib.ycm_create(page_size, n, pages, wins, num_slots)
+        keep = (ctypes.c_int32 * max(n, 1))(*[int(g.keep_first or 0) for g in self.groups])
+        self.h = self.lib.ycm_create(page_size, n, pages, wins, keep, num_slots)
         if not self.h:
             raise CacheError(self.lib.ycm_last_error().decode())
 

@@ -51,8 +51,10 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_of(raw: Dict[str, Any]) -> Architecture:
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str):
+        return get_architecture(raw["architecture"])  # some families name themselves with one string
     if not isinstance(archs, list) or len(archs) < 1 or not isinstance(archs[0], str):
-        raise ConfigError("config.json: 'architectures' must be a list holding the model class name")
+        raise ConfigError("config.json: 'architectures' must be a list holding the model class name (or 'architecture' a string)")
     return get_architecture(archs[0])
 
 

@@ -1,0 +1,353 @@
+// Attention whose heads are prepared, masked and finished in more ways than the plain causal one:
+//
+//  * yk_qkv_prepare: what happens to a projection's rows [q heads | k heads | v heads | ...]
+//    before the scores: an RMS norm per head on queries and keys (a weight of head_dim elements
+//    shared by the heads, or none), rotary positions on the first rotary_dim elements of queries
+//    and keys, values divided by their root mean square per head, values rotated by their own
+//    table over all of value_dim; queries go to a tensor, keys and values into the pages.
+//    Every option can be left out; with none of them it is rotary + append.
+//  * yk_attn_masked: scores q . k * scale, optionally squashed s <- cap * tanh(s / cap); key j
+//    is visible to the query at position p iff j <= p and (p - j < window or j < keep_first)
+//    (window 0: no window); softmax over the visible keys; keys of head_dim, values of
+//    value_dim elements.  One wave per (token, head), float32 arithmetic, any sizes up to 256.
+//    Its epilogue can turn the output back by the query's own position (the inverse of the
+//    values' rotation) and multiply a head's output by the sigmoid of a gate column of the
+//    projection.
+//  * yk_attn_finish: that epilogue alone, in place, for outputs that another attention kernel made.
+//
+// Norms, angles, scores, softmax and the gate are float32; values are rounded once when stored.
+#include <algorithm>
+
+#include "common.h"
+
+namespace {
+
+constexpr int kMaxHead = 256;
+
+// Rotate the first `rot` elements of buf[0..len) (float32, in LDS) by the angles of `pos`;
+// lane's elements are lane, lane + 64, ...  `sign` -1 turns the other way.
+__device__ __forceinline__ float rotated_element(const float* buf, int i, int rot, int interleaved,
+                                                 const float* __restrict__ cos_row,
+                                                 const float* __restrict__ sin_row, float sign) {
+  if (i >= rot) return buf[i];
+  if (interleaved) {
+    const int m = i / 2;
+    const float c = cos_row[m], s = sign * sin_row[m];
+    return (i % 2 == 0) ? rot_first(buf[i], buf[i + 1], c, s) : rot_second(buf[i - 1], buf[i], c, s);
+  }
+  const int half = rot / 2;
+  if (i < half) return rot_first(buf[i], buf[i + half], cos_row[i], sign * sin_row[i]);
+  return rot_second(buf[i - half], buf[i], cos_row[i - half], sign * sin_row[i - half]);
+}
+
+}  // namespace
+
+template <typename TS, typename T, typename TW>
+__global__ __launch_bounds__(64) void qkv_prepare_kernel(
+    const TS* __restrict__ src, int n_splits, size_t split_stride, int round_sum, int src_stride,
+    T* __restrict__ q_out, int q_stride, int n_heads, int n_kv, int head_dim, int v_dim,
+    const int32_t* __restrict__ positions, const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w,
+    int qk_norm, float qk_eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim,
+    int interleaved, int max_pos, int v_norm, float v_eps, const float* __restrict__ v_cos,
+    const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size, int tiled) {
+  __shared__ float buf[kMaxHead];
+  const int n = blockIdx.x, slot_y = blockIdx.y, lane = threadIdx.x;
+  const int kind = slot_y < n_heads ? 0 : (slot_y < n_heads + n_kv ? 1 : 2);  // q, k, v
+  const int len = kind == 2 ? v_dim : head_dim;
+  int col0;
+  if (kind == 0) col0 = slot_y * head_dim;
+  else if (kind == 1) col0 = n_heads * head_dim + (slot_y - n_heads) * head_dim;
+  else col0 = (n_heads + n_kv) * head_dim + (slot_y - n_heads - n_kv) * v_dim;
+  const TS* row = src + static_cast<size_t>(n) * src_stride + col0;
+  float val[4];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    float v = 0.f;
+    if (d < len) {
+      for (int s = 0; s < n_splits; ++s) v += to_f32<TS>(row[s * split_stride + d]);
+      v = as_output(v, round_sum);
+    }
+    val[i] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const bool normed = kind == 2 ? v_norm != 0 : qk_norm != 0;
+  if (normed) {
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(len) + (kind == 2 ? v_eps : qk_eps));
+    const TW* w = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < len) val[i] = val[i] * inv * (w != nullptr ? to_f32<TW>(w[d]) : 1.f);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < len) buf[d] = val[i];
+  }
+  __syncthreads();
+  const int pos = positions[n];
+  const float *cr = nullptr, *sr = nullptr;
+  int rot = 0, inter = 0;
+  if (kind == 2) {
+    if (v_cos != nullptr) {
+      const int p = min(pos, v_max_pos - 1);
+      rot = v_dim, inter = v_interleaved;
+      cr = v_cos + static_cast<size_t>(p) * (v_dim / 2);
+      sr = v_sin + static_cast<size_t>(p) * (v_dim / 2);
+    }
+  } else if (rotary_dim > 0) {
+    const int p = min(pos, max_pos - 1);
+    rot = rotary_dim, inter = interleaved;
+    cr = cos_t + static_cast<size_t>(p) * (rotary_dim / 2);
+    sr = sin_t + static_cast<size_t>(p) * (rotary_dim / 2);
+  }
+  size_t base = 0;
+  int off = 0;
+  if (kind != 0) {
+    const int slot = slots[n];
+    const int page = slot / page_size, g = kind == 1 ? slot_y - n_heads : slot_y - n_heads - n_kv;
+    off = slot % page_size;
+    base = (static_cast<size_t>(page) * n_kv + g) * page_size * (kind == 1 ? head_dim : v_dim);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d >= len) continue;
+    const float v = rot > 0 ? rotated_element(buf, d, rot, inter, cr, sr, 1.f) : buf[d];
+    if (kind == 0)
+      q_out[static_cast<size_t>(n) * q_stride + col0 + d] = from_f32<T>(v);
+    else if (kind == 1)
+      k_cache[base + cache_k_offset(tiled, page_size, head_dim, off, d)] = from_f32<T>(v);
+    else
+      v_cache[base + cache_v_offset(tiled, page_size, v_dim, off, d)] = from_f32<T>(v);
+  }
+}
+
+extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int round_sum, int src_stride, void* q_out,
+                              int act_dtype, int q_stride, int n_tokens, int n_heads, int n_kv, int head_dim, int v_dim,
+                              const int32_t* positions, const void* q_norm_w, const void* k_norm_w, int norm_w_dtype,
+                              int qk_norm, float qk_eps, const float* cos_t, const float* sin_t, int rotary_dim,
+                              int interleaved, int max_pos, int v_norm, float v_eps, const float* v_cos,
+                              const float* v_sin, int v_interleaved, int v_max_pos, void* k_cache, void* v_cache,
+                              const int32_t* slots, int page_size, int tiled, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv >= 0, "qkv_prepare: bad sizes");
+  YK_REQUIRE(head_dim > 0 && head_dim <= kMaxHead && v_dim > 0 && v_dim <= kMaxHead, "qkv_prepare: heads of 1 to 256 elements");
+  YK_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "qkv_prepare: rotary_dim must be even and at most head_dim");
+  YK_REQUIRE(rotary_dim == 0 || (cos_t != nullptr && sin_t != nullptr && max_pos > 0), "qkv_prepare: rotary tables missing");
+  YK_REQUIRE(v_cos == nullptr || (v_sin != nullptr && v_max_pos > 0 && v_dim % 2 == 0), "qkv_prepare: value tables need an even value_dim");
+  YK_REQUIRE(n_kv == 0 || (k_cache != nullptr && v_cache != nullptr && slots != nullptr && page_size > 0), "qkv_prepare: no pages to append to");
+  YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "qkv_prepare: unreduced slices must be float32");
+  YK_REQUIRE(!tiled || (head_dim == v_dim && cache_is_tiled(act_dtype, head_dim, page_size)), "qkv_prepare: these pages cannot be tiled");
+  YK_REQUIRE(n_heads + 2 * n_kv <= 65535, "qkv_prepare: too many heads for one launch");
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, n_heads + 2 * n_kv), block(64);
+  const size_t stride = static_cast<size_t>(n_tokens) * src_stride;
+#define YK_CASE(SD, TS, AD, T, WD, TW)                                                                       \
+  if (src_dtype == SD && act_dtype == AD && (norm_w_dtype == WD || (q_norm_w == nullptr && k_norm_w == nullptr && WD == YK_F32))) { \
+    qkv_prepare_kernel<TS, T, TW><<<grid, block, 0, stream>>>(                                                \
+        static_cast<const TS*>(src), n_splits, stride, round_sum, src_stride, static_cast<T*>(q_out), q_stride,  \
+        n_heads, n_kv, head_dim, v_dim, positions, static_cast<const TW*>(q_norm_w),                          \
+        static_cast<const TW*>(k_norm_w), qk_norm, qk_eps, cos_t, sin_t, rotary_dim, interleaved, max_pos,     \
+        v_norm, v_eps, v_cos, v_sin, v_interleaved, v_max_pos, static_cast<T*>(k_cache), static_cast<T*>(v_cache), \
+        slots, page_size, tiled);                                                                             \
+    return yk_check_launch("qkv_prepare");                                                                    \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_BF16, bf16_t)
+#undef YK_CASE
+  return yk_fail("qkv_prepare: unsupported dtype combination");
+}
+
+// ------------------------------------------------------------------------------ the finish
+// One head's output `os` [v_dim] (float32, LDS), turned back by the position and gated.
+template <typename TG>
+__device__ __forceinline__ float head_gate(const TG* __restrict__ gate_src, int gate_splits, size_t gate_split_stride,
+                                           int gate_round, size_t index) {
+  float g = 0.f;
+  for (int s = 0; s < gate_splits; ++s) g += to_f32<TG>(gate_src[s * gate_split_stride + index]);
+  g = as_output(g, gate_round);
+  return 1.f / (1.f + expf(-g));
+}
+
+template <typename T, typename TG>
+__global__ __launch_bounds__(64) void attn_masked_kernel(
+    const T* __restrict__ q, int q_stride, T* __restrict__ out, const T* __restrict__ k_cache,
+    const T* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ token_seq,
+    const int32_t* __restrict__ block_table, int table_width, int page_size, int head_dim, int v_dim, int n_heads,
+    int n_kv, float scale, float softcap, int window, int keep_first, int tiled, const float* __restrict__ v_cos,
+    const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, const TG* __restrict__ gate_src,
+    int gate_splits, size_t gate_split_stride, int gate_round, int gate_stride, int gate_col0) {
+  const size_t slab_k = static_cast<size_t>(page_size) * head_dim, slab_v = static_cast<size_t>(page_size) * v_dim;
+  __shared__ float qs[kMaxHead];
+  __shared__ float os[kMaxHead];
+  __shared__ float ps[64];
+  __shared__ int pbase[64];  // (page * n_kv + kv_head) per key of the tile
+  __shared__ int poff[64];
+  const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int qpk = n_heads / n_kv, g = h / qpk;
+  const int pos = positions[n], seq = token_seq[n];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int n_first = min(keep_first, lo);  // keys below the window that stay visible
+  const int total = n_first + (pos + 1 - lo);
+  const T* qrow = q + static_cast<size_t>(n) * q_stride + static_cast<size_t>(h) * head_dim;
+  for (int d = lane; d < head_dim; d += 64) qs[d] = to_f32<T>(qrow[d]);
+  __syncthreads();
+  const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
+  float m = -INFINITY, l = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = 0; t0 < total; t0 += 64) {
+    const int idx = t0 + lane;
+    const bool valid = idx < total;
+    float s = -INFINITY;
+    int base = 0, off = 0;
+    if (valid) {
+      const int key = idx < n_first ? idx : lo + (idx - n_first);
+      const int page = bt[key / page_size];
+      off = key % page_size;
+      base = page * n_kv + g;
+      const T* kp = k_cache + static_cast<size_t>(base) * slab_k;
+      float dot = 0.f;
+      for (int d = 0; d < head_dim; ++d)
+        dot = fmaf(qs[d], to_f32<T>(kp[cache_k_offset(tiled, page_size, head_dim, off, d)]), dot);
+      s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+    }
+    const float m_new = fmaxf(m, wave_max(s));  // finite: the tile holds at least one key
+    const float p = valid ? expf(s - m_new) : 0.f;
+    const float alpha = expf(m - m_new);  // 0 on the first tile
+    l = l * alpha + wave_sum(p);
+    m = m_new;
+    __syncthreads();  // the previous tile's ps/pbase are no longer read
+    ps[lane] = p;
+    pbase[lane] = base;
+    poff[lane] = off;
+    __syncthreads();
+    const int count = min(64, total - t0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < v_dim) {
+        float a = acc[i] * alpha;
+        for (int j = 0; j < count; ++j) {
+          const T* vp = v_cache + static_cast<size_t>(pbase[j]) * slab_v + cache_v_offset(tiled, page_size, v_dim, poff[j], d);
+          a = fmaf(ps[j], to_f32<T>(*vp), a);
+        }
+        acc[i] = a;
+      }
+    }
+  }
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < v_dim) os[d] = acc[i] * inv;
+  }
+  __syncthreads();
+  float gate = 1.f;
+  if (gate_src != nullptr)
+    gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, static_cast<size_t>(n) * gate_stride + gate_col0 + h);
+  const float *cr = nullptr, *sr = nullptr;
+  if (v_cos != nullptr) {
+    const int p = min(pos, v_max_pos - 1);
+    cr = v_cos + static_cast<size_t>(p) * (v_dim / 2);
+    sr = v_sin + static_cast<size_t>(p) * (v_dim / 2);
+  }
+  T* orow = out + (static_cast<size_t>(n) * n_heads + h) * v_dim;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < v_dim) {
+      const float v = cr != nullptr ? rotated_element(os, d, v_dim, v_interleaved, cr, sr, -1.f) : os[d];
+      orow[d] = from_f32<T>(v * gate);
+    }
+  }
+}
+
+extern "C" int yk_attn_masked(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache, int dtype,
+                              const int32_t* positions, const int32_t* token_seq, const int32_t* block_table,
+                              int table_width, int n_tokens, int page_size, int head_dim, int v_dim, int n_heads, int n_kv,
+                              float scale, float softcap, int window, int keep_first, int tiled, const float* v_cos,
+                              const float* v_sin, int v_interleaved, int v_max_pos, const void* gate_src, int gate_dtype,
+                              int gate_splits, int gate_round, int gate_stride, int gate_col0, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_masked: bad head counts");
+  YK_REQUIRE(head_dim > 0 && head_dim <= kMaxHead && v_dim > 0 && v_dim <= kMaxHead, "attn_masked: heads of 1 to 256 elements");
+  YK_REQUIRE(page_size > 0 && table_width > 0, "attn_masked: bad page table");
+  YK_REQUIRE(window >= 0 && keep_first >= 0 && softcap >= 0.f, "attn_masked: window, keep_first and softcap must not be negative");
+  YK_REQUIRE(n_heads <= 65535, "attn_masked: too many heads for one launch");
+  YK_REQUIRE(v_cos == nullptr || (v_sin != nullptr && v_max_pos > 0 && v_dim % 2 == 0), "attn_masked: value tables need an even value_dim");
+  YK_REQUIRE(!tiled || (head_dim == v_dim && cache_is_tiled(dtype, head_dim, page_size)), "attn_masked: these pages cannot be tiled");
+  YK_REQUIRE(gate_src == nullptr || gate_splits >= 1, "attn_masked: bad gate");
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, n_heads), block(64);
+  const size_t gstride = static_cast<size_t>(n_tokens) * gate_stride;
+#define YK_CASE(D, T, GD, TG)                                                                                 \
+  if (dtype == D && (gate_src == nullptr ? GD == D : gate_dtype == GD)) {                                      \
+    attn_masked_kernel<T, TG><<<grid, block, 0, stream>>>(                                                     \
+        static_cast<const T*>(q), q_stride, static_cast<T*>(out), static_cast<const T*>(k_cache),              \
+        static_cast<const T*>(v_cache), positions, token_seq, block_table, table_width, page_size, head_dim,   \
+        v_dim, n_heads, n_kv, scale, softcap, window, keep_first, tiled, v_cos, v_sin, v_interleaved, v_max_pos, \
+        static_cast<const TG*>(gate_src), gate_splits, gstride, gate_round, gate_stride, gate_col0);           \
+    return yk_check_launch("attn_masked");                                                                     \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
+#undef YK_CASE
+  return yk_fail("attn_masked: unsupported dtype combination");
+}
+
+template <typename T, typename TG>
+__global__ __launch_bounds__(64) void attn_finish_kernel(
+    T* __restrict__ out, const int32_t* __restrict__ positions, int v_dim, int n_heads, const float* __restrict__ v_cos,
+    const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, const TG* __restrict__ gate_src, int gate_splits,
+    size_t gate_split_stride, int gate_round, int gate_stride, int gate_col0) {
+  __shared__ float os[kMaxHead];
+  const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  T* orow = out + (static_cast<size_t>(n) * n_heads + h) * v_dim;
+  for (int d = lane; d < v_dim; d += 64) os[d] = to_f32<T>(orow[d]);
+  __syncthreads();
+  float gate = 1.f;
+  if (gate_src != nullptr)
+    gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, static_cast<size_t>(n) * gate_stride + gate_col0 + h);
+  const float *cr = nullptr, *sr = nullptr;
+  if (v_cos != nullptr) {
+    const int p = min(positions[n], v_max_pos - 1);
+    cr = v_cos + static_cast<size_t>(p) * (v_dim / 2);
+    sr = v_sin + static_cast<size_t>(p) * (v_dim / 2);
+  }
+  for (int d = lane; d < v_dim; d += 64) {
+    const float v = cr != nullptr ? rotated_element(os, d, v_dim, v_interleaved, cr, sr, -1.f) : os[d];
+    orow[d] = from_f32<T>(v * gate);
+  }
+}
+
+extern "C" int yk_attn_finish(void* out, int dtype, const int32_t* positions, int n_tokens, int v_dim, int n_heads,
+                              const float* v_cos, const float* v_sin, int v_interleaved, int v_max_pos,
+                              const void* gate_src, int gate_dtype, int gate_splits, int gate_round, int gate_stride,
+                              int gate_col0, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_heads <= 65535 && v_dim > 0 && v_dim <= kMaxHead, "attn_finish: bad sizes");
+  YK_REQUIRE(v_cos == nullptr || (v_sin != nullptr && v_max_pos > 0 && v_dim % 2 == 0), "attn_finish: value tables need an even value_dim");
+  if (n_tokens == 0 || (v_cos == nullptr && gate_src == nullptr)) return 0;
+  dim3 grid(n_tokens, n_heads), block(64);
+  const size_t gstride = static_cast<size_t>(n_tokens) * gate_stride;
+#define YK_CASE(D, T, GD, TG)                                                                          \
+  if (dtype == D && (gate_src == nullptr ? GD == D : gate_dtype == GD)) {                               \
+    attn_finish_kernel<T, TG><<<grid, block, 0, stream>>>(static_cast<T*>(out), positions, v_dim, n_heads, v_cos, v_sin, \
+                                                          v_interleaved, v_max_pos, static_cast<const TG*>(gate_src),   \
+                                                          gate_splits, gstride, gate_round, gate_stride, gate_col0);    \
+    return yk_check_launch("attn_finish");                                                              \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
+#undef YK_CASE
+  return yk_fail("attn_finish: unsupported dtype combination");
+}

@@ -27,6 +27,7 @@ namespace {
 struct Group {
   int32_t num_pages = 0;
   int32_t window = 0;  // 0: keep everything
+  int32_t keep_first = 0;  // with a window: the first tokens that stay readable (their pages are never given back)
   std::deque<int32_t> free_pages;
 };
 
@@ -64,9 +65,10 @@ extern "C" {
 
 const char* ycm_last_error() { return g_error.c_str(); }
 
-// windows[g] == 0 means the group keeps every token.
+// windows[g] == 0 means the group keeps every token; keep_first[g] tokens at the start of every
+// request stay whatever the window says (keep_first may be null: none).
 void* ycm_create(int32_t page_size, int32_t num_groups, const int32_t* num_pages,
-                 const int32_t* windows, int32_t num_slots) {
+                 const int32_t* windows, const int32_t* keep_first, int32_t num_slots) {
   if (page_size <= 0 || num_groups < 0 || num_slots <= 0) {
     g_error = "ycm_create: page_size and num_slots must be positive";
     return nullptr;
@@ -77,13 +79,14 @@ void* ycm_create(int32_t page_size, int32_t num_groups, const int32_t* num_pages
   for (int32_t s = 0; s < num_slots; ++s) m->free_slots.insert(s);
   m->groups.resize(num_groups);
   for (int32_t g = 0; g < num_groups; ++g) {
-    if (num_pages[g] <= 0 || windows[g] < 0) {
-      g_error = "ycm_create: a group needs pages and a non-negative window";
+    if (num_pages[g] <= 0 || windows[g] < 0 || (keep_first && keep_first[g] < 0)) {
+      g_error = "ycm_create: a group needs pages, a non-negative window and a non-negative count of kept first tokens";
       delete m;
       return nullptr;
     }
     m->groups[g].num_pages = num_pages[g];
     m->groups[g].window = windows[g];
+    m->groups[g].keep_first = keep_first ? keep_first[g] : 0;
     for (int32_t p = 0; p < num_pages[g]; ++p) m->groups[g].free_pages.push_back(p);
   }
   return m;
@@ -150,7 +153,8 @@ int32_t ycm_reserve(void* h, int64_t req, int64_t total_tokens) {
 }
 
 // After a step: cached_tokens of the request are in the cache.  Groups with a
-// window give back every page that no later token can read: the next query sits
+// window give back every page that no later token can read (but never a page with one of
+// the group's kept first tokens): the next query sits
 // at position >= cached_tokens and reads keys j with position - j < window, so
 // keys j <= cached_tokens - window are dead.  Returns the number of pages freed.
 int32_t ycm_advance(void* h, int64_t req, int64_t cached_tokens) {
@@ -166,7 +170,9 @@ int32_t ycm_advance(void* h, int64_t req, int64_t cached_tokens) {
     if (dead_tokens <= 0) continue;
     int64_t dead_pages = dead_tokens / m->page_size;  // whole pages only
     dead_pages = std::min<int64_t>(dead_pages, static_cast<int64_t>(r.tables[g].size()));
-    for (int64_t p = r.first_live[g]; p < dead_pages; ++p) {
+    // pages that hold any of the kept first tokens stay
+    const int64_t kept_pages = pages_for(m->groups[g].keep_first, m->page_size);
+    for (int64_t p = std::max(r.first_live[g], kept_pages); p < dead_pages; ++p) {
       int32_t page = r.tables[g][p];
       if (page >= 0) {
         m->groups[g].free_pages.push_back(page);

@@ -138,6 +138,16 @@ __device__ __forceinline__ float act_gelu_tanh(float z) {
   return 0.5f * z * (1.f + tanhf(k * (z + 0.044715f * z * z * z)));
 }
 __device__ __forceinline__ float act_apply(float z, int act) { return act == 0 ? act_silu(z) : act_gelu_tanh(z); }
+// A gated pair: what a feed-forward makes of a gate value g and an up value u.  Kinds 0 and 1:
+// act(g) * u.  Kind 2, the clamped swish gate: g' = min(g, p0), u' = clamp(u, -p0, p0),
+// g' * sigmoid(p1 * g') * (u' + 1) (p0 the limit, p1 the slope of the sigmoid).
+#define YK_GATED_KINDS 3
+__device__ __forceinline__ float gated_pair(float g, float u, int kind, float p0, float p1) {
+  if (kind < 2) return act_apply(g, kind) * u;
+  g = fminf(g, p0);
+  u = fminf(fmaxf(u, -p0), p0);
+  return g / (1.f + expf(-p1 * g)) * (u + 1.f);
+}
 
 // The sum of a product's K slices (or an accumulator) stands for the product's output: with
 // `round_sum` it is rounded to bfloat16 as that output would have been, so that what follows

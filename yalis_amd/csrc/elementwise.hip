@@ -587,7 +587,7 @@ __device__ __forceinline__ size_t up_offset(int inter, int group) { return group
 
 template <typename TS, typename TO>
 __global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride, int round_sum,
-                                 TO* __restrict__ out, int inter, size_t total, int act, int group) {
+                                 TO* __restrict__ out, int inter, size_t total, int act, int group, float p0, float p1) {
   for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const size_t n = i / inter, j = i % inter;
@@ -599,14 +599,14 @@ __global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t
     }
     g = as_output(g, round_sum);
     u = as_output(u, round_sum);
-    out[i] = from_f32<TO>(act_apply(g, act) * u);
+    out[i] = from_f32<TO>(gated_pair(g, u, act, p0, p1));
   }
 }
 
 // four outputs per thread, no loop (inter a multiple of 4)
 template <typename TS, typename TO>
 __global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride, int round_sum,
-                                     TO* __restrict__ out, int inter, size_t total_vec, int act, int group) {
+                                     TO* __restrict__ out, int inter, size_t total_vec, int act, int group, float p0, float p1) {
   const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
   if (v >= total_vec) return;
   const int per_row = inter / 4;
@@ -627,17 +627,17 @@ __global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, si
     }
   }
   float4 y;
-  y.x = act_apply(as_output(g.x, round_sum), act) * as_output(u.x, round_sum);
-  y.y = act_apply(as_output(g.y, round_sum), act) * as_output(u.y, round_sum);
-  y.z = act_apply(as_output(g.z, round_sum), act) * as_output(u.z, round_sum);
-  y.w = act_apply(as_output(g.w, round_sum), act) * as_output(u.w, round_sum);
+  y.x = gated_pair(as_output(g.x, round_sum), as_output(u.x, round_sum), act, p0, p1);
+  y.y = gated_pair(as_output(g.y, round_sum), as_output(u.y, round_sum), act, p0, p1);
+  y.z = gated_pair(as_output(g.z, round_sum), as_output(u.z, round_sum), act, p0, p1);
+  y.w = gated_pair(as_output(g.w, round_sum), as_output(u.w, round_sum), act, p0, p1);
   store4<TO>(out + n * inter + j, y);
 }
 
 // bfloat16 in and out, one slice, eight outputs per thread with 16-byte accesses (in the
 // grouped layout a thread's gate and up values are 32 contiguous bytes)
 __global__ void gated_act_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int inter,
-                                        size_t total_vec, int act, int group) {
+                                        size_t total_vec, int act, int group, float p0, float p1) {
   const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
   if (v >= total_vec) return;
   const int per_row = inter / 8;
@@ -652,14 +652,14 @@ __global__ void gated_act_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* _
   for (int k = 0; k < 4; ++k) {
     const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
     const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
-    o[k] = pack_bf16x2(act_apply(g0, act) * u0, act_apply(g1, act) * u1);
+    o[k] = pack_bf16x2(gated_pair(g0, u0, act, p0, p1), gated_pair(g1, u1, act, p0, p1));
   }
   *reinterpret_cast<uint4*>(out + n * inter + j) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 template <typename TS, typename TO>
 static int launch_gated_act(const void* gu, int n_splits, int round_sum, void* out, int n_rows, int inter, int act,
-                            int group, hipStream_t stream) {
+                            int group, float p0, float p1, hipStream_t stream) {
   const size_t stride = static_cast<size_t>(n_rows) * 2 * inter;
   const bool aligned = inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0;
@@ -667,31 +667,31 @@ static int launch_gated_act(const void* gu, int n_splits, int round_sum, void* o
     const size_t total_vec = static_cast<size_t>(n_rows) * (inter / 8);
     YK_REQUIRE((total_vec + 255) / 256 < (1ull << 31), "gated_act: too large for one launch");
     gated_act_bf16x8_kernel<<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
-        static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), inter, total_vec, act, group);
+        static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), inter, total_vec, act, group, p0, p1);
   } else if (aligned) {
     const size_t total_vec = static_cast<size_t>(n_rows) * (inter / 4);
     YK_REQUIRE((total_vec + 255) / 256 < (1ull << 31), "gated_act: too large for one launch");
     gated_act_vec_kernel<TS, TO><<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
-        static_cast<const TS*>(gu), n_splits, stride, round_sum, static_cast<TO*>(out), inter, total_vec, act, group);
+        static_cast<const TS*>(gu), n_splits, stride, round_sum, static_cast<TO*>(out), inter, total_vec, act, group, p0, p1);
   } else {
     const size_t total = static_cast<size_t>(n_rows) * inter;
     const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 65535));
     gated_act_kernel<TS, TO><<<grid, 256, 0, stream>>>(static_cast<const TS*>(gu), n_splits, stride, round_sum,
-                                                        static_cast<TO*>(out), inter, total, act, group);
+                                                        static_cast<TO*>(out), inter, total, act, group, p0, p1);
   }
   return yk_check_launch("gated_act");
 }
 
 extern "C" int yk_gated_act(const void* gu, int src_dtype, int n_splits, int round_sum, void* out, int out_dtype,
-                            int n_rows, int inter, int act, int group, hipStream_t stream) {
+                            int n_rows, int inter, int act, int group, float p0, float p1, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && inter > 0, "gated_act: bad sizes");
   YK_REQUIRE(group == 0 || (group % 4 == 0 && inter % group == 0), "gated_act: groups are multiples of 4 that divide the width");
-  YK_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation");
+  YK_REQUIRE(act >= 0 && act < YK_GATED_KINDS, "gated_act: unknown activation");
   YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "gated_act: unreduced slices must be float32");
   if (n_rows == 0) return 0;
-  if (src_dtype == YK_F32 && out_dtype == YK_F32) return launch_gated_act<float, float>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
-  if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
-  if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
+  if (src_dtype == YK_F32 && out_dtype == YK_F32) return launch_gated_act<float, float>(gu, n_splits, round_sum, out, n_rows, inter, act, group, p0, p1, stream);
+  if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, p0, p1, stream);
+  if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, p0, p1, stream);
   return yk_fail("gated_act: unsupported dtype combination");
 }
 

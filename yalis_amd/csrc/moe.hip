@@ -1,0 +1,300 @@
+// A mixture of small gated feed-forward experts over a ragged batch of tokens.
+//
+// Which experts a token uses is decided before these kernels (by a table over token ids here;
+// a learned router would write the same arrays): `choice` [tokens, top] names them.  A (token,
+// k-th choice) is a "pair", numbered token * top + k.
+//   * moe_route: sorts the pairs by expert (a counting sort in one workgroup) and cuts every
+//     expert's run into tiles of `tile_rows` pairs: order [pairs], slot_expert [pairs], and a
+//     tile list (expert, first sorted slot, count).  The order of the pairs inside a run is
+//     whatever the atomics gave; every pair's row is computed on its own, so no result depends
+//     on it.
+//   * moe_gate_up: for the pair in sorted slot i with expert e, y[i, :] = gated_pair(x[token] .
+//     Wg_e^T, x[token] . Wu_e^T); the weights of all experts are one tensor [experts][2][ff][hidden].
+//   * moe_down: rows[pair, :] = y[i, :] . Wd_e^T in float32, stored in pair order (token-major), so
+//     that whoever adds a token's rows finds them side by side (the norm that follows does).
+// Each product has a float32 FMA form for any sizes and dtypes, and a matrix-core form for
+// bfloat16 with K a multiple of 32: a wave multiplies 16 weight rows (the A operand, straight
+// from memory) with 16 * MT pairs (the B operand, gathered rows of x), so an expert's weights are
+// read once per tile of pairs.
+#include <algorithm>
+
+#include "common.h"
+
+// ------------------------------------------------------------------------------- routing
+__global__ __launch_bounds__(1024) void moe_route_kernel(
+    const int32_t* __restrict__ token_ids, const int32_t* __restrict__ table, int vocab, int top, int n_experts,
+    int n_pairs, int tile_rows, int32_t* __restrict__ order, int32_t* __restrict__ slot_expert,
+    int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles_out, int max_tiles) {
+  extern __shared__ int lds[];  // [n_experts] counts, then cursors; [n_experts + 1] first tile of each expert
+  int* cnt = lds;
+  int* tile0 = lds + n_experts;
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
+    int id = token_ids[i / top];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const int e = table[static_cast<size_t>(id) * top + i % top];
+    atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0, t = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      const int c = cnt[e];
+      tile0[e] = t;
+      t += (c + tile_rows - 1) / tile_rows;
+      cnt[e] = run;  // becomes the cursor
+      run += c;
+    }
+    tile0[n_experts] = t;
+    *n_tiles_out = t < max_tiles ? t : max_tiles;
+  }
+  __syncthreads();
+  // the tiles of every expert, from the run starts that the cursors still hold
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    const int first = cnt[e];
+    const int n_t = tile0[e + 1] - tile0[e];
+    const int len = (e + 1 < n_experts ? cnt[e + 1] : n_pairs) - first;  // starts are running sums
+    for (int k = 0; k < n_t; ++k) {
+      const int t = tile0[e] + k;
+      if (t < max_tiles) {
+        tiles[3 * t] = e;
+        tiles[3 * t + 1] = first + k * tile_rows;
+        tiles[3 * t + 2] = min(tile_rows, len - k * tile_rows);
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
+    int id = token_ids[i / top];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const int e = table[static_cast<size_t>(id) * top + i % top];
+    const int at = atomicAdd(&cnt[e], 1);
+    order[at] = i;
+    slot_expert[at] = e;
+  }
+}
+
+extern "C" int yk_moe_max_tiles(int n_pairs, int n_experts, int tile_rows) {
+  return (n_pairs + tile_rows - 1) / tile_rows + n_experts;
+}
+
+extern "C" int yk_moe_route(const int32_t* token_ids, const int32_t* table, int vocab, int top, int n_experts,
+                            int n_tokens, int tile_rows, int32_t* order, int32_t* slot_expert, int32_t* tiles,
+                            int32_t* n_tiles, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && top >= 1 && n_experts >= 1 && vocab >= 1 && tile_rows >= 1, "moe_route: bad sizes");
+  YK_REQUIRE(n_experts <= 4096, "moe_route: more than 4,096 experts");
+  if (n_tokens == 0) return 0;
+  const int n_pairs = n_tokens * top;
+  const size_t lds = (2 * static_cast<size_t>(n_experts) + 1) * sizeof(int);
+  moe_route_kernel<<<1, 1024, lds, stream>>>(token_ids, table, vocab, top, n_experts, n_pairs, tile_rows, order,
+                                             slot_expert, tiles, n_tiles, yk_moe_max_tiles(n_pairs, n_experts, tile_rows));
+  return yk_check_launch("moe_route");
+}
+
+// ---------------------------------------------------------------- float32 FMA products
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void moe_gate_up_fma_kernel(
+    const T* __restrict__ x, int x_stride, const TW* __restrict__ w, const int32_t* __restrict__ order,
+    const int32_t* __restrict__ slot_expert, int top, int hidden, int ff, int kind, float p0, float p1,
+    T* __restrict__ y) {
+  extern __shared__ float xs[];  // [hidden]
+  const int i = blockIdx.x;
+  const int token = order[i] / top, e = slot_expert[i];
+  for (int k = threadIdx.x; k < hidden; k += blockDim.x) xs[k] = to_f32<T>(x[static_cast<size_t>(token) * x_stride + k]);
+  __syncthreads();
+  for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < ff; j += gridDim.y * blockDim.x) {
+    const TW* wg = w + (static_cast<size_t>(e) * 2 * ff + j) * hidden;
+    const TW* wu = wg + static_cast<size_t>(ff) * hidden;
+    float g = 0.f, u = 0.f;
+    for (int k = 0; k < hidden; ++k) {
+      g = fmaf(to_f32<TW>(wg[k]), xs[k], g);
+      u = fmaf(to_f32<TW>(wu[k]), xs[k], u);
+    }
+    y[static_cast<size_t>(i) * ff + j] = from_f32<T>(gated_pair(g, u, kind, p0, p1));
+  }
+}
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void moe_down_fma_kernel(
+    const T* __restrict__ y, const TW* __restrict__ w, const int32_t* __restrict__ order,
+    const int32_t* __restrict__ slot_expert, int hidden, int ff, float* __restrict__ rows) {
+  extern __shared__ float ys[];  // [ff]
+  const int i = blockIdx.x;
+  const int pair = order[i], e = slot_expert[i];
+  for (int k = threadIdx.x; k < ff; k += blockDim.x) ys[k] = to_f32<T>(y[static_cast<size_t>(i) * ff + k]);
+  __syncthreads();
+  for (int h = blockIdx.y * blockDim.x + threadIdx.x; h < hidden; h += gridDim.y * blockDim.x) {
+    const TW* wd = w + (static_cast<size_t>(e) * hidden + h) * ff;
+    float acc = 0.f;
+    for (int k = 0; k < ff; ++k) acc = fmaf(to_f32<TW>(wd[k]), ys[k], acc);
+    rows[static_cast<size_t>(pair) * hidden + h] = acc;
+  }
+}
+
+// ---------------------------------------------------------------- matrix-core products
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+union MoeFrag {
+  u32x4_t u;
+  bf16x8_t v;
+};
+
+// Operands of v_mfma_f32_16x16x32_bf16 (r = lane % 16, g = lane / 16): A lane holds A[r][8g..8g+7],
+// B lane holds B[8g..8g+7][r], C lane holds C[4g..4g+3][r].  A = 16 weight rows, B = 16 pairs'
+// rows of x: C[i][r] = (pair r, feature 4g + i).
+template <int MT>
+__global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
+    const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
+    const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, int top, int hidden, int ff, int kind,
+    float p0, float p1, bf16_t* __restrict__ y) {
+  const int t = blockIdx.x;
+  if (t >= *n_tiles) return;
+  const int e = tiles[3 * t], first = tiles[3 * t + 1], count = tiles[3 * t + 2];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r = lane % 16, g = lane / 16;
+  const int f0 = (blockIdx.y * 4 + wave) * 16;
+  if (f0 >= ff) return;
+  const bf16_t* wg = w + (static_cast<size_t>(e) * 2 * ff + f0 + r) * hidden + 8 * g;
+  const bf16_t* wu = wg + static_cast<size_t>(ff) * hidden;
+  const bf16_t* xr[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int slot = first + min(16 * m + r, count - 1);  // rows beyond the tile repeat its last pair and are not stored
+    xr[m] = x + static_cast<size_t>(order[slot] / top) * x_stride + 8 * g;
+  }
+  f32x4_t ag[MT], au[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) ag[m] = au[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < hidden; k0 += 32) {
+    MoeFrag a_g, a_u, b[MT];
+    a_g.u = *reinterpret_cast<const u32x4_t*>(wg + k0);
+    a_u.u = *reinterpret_cast<const u32x4_t*>(wu + k0);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) b[m].u = *reinterpret_cast<const u32x4_t*>(xr[m] + k0);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      ag[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_g.v, b[m].v, ag[m], 0, 0, 0);
+      au[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_u.v, b[m].v, au[m], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    if (16 * m + r < count) {
+      uint32_t o[2];
+      o[0] = pack_bf16x2(gated_pair(ag[m][0], au[m][0], kind, p0, p1), gated_pair(ag[m][1], au[m][1], kind, p0, p1));
+      o[1] = pack_bf16x2(gated_pair(ag[m][2], au[m][2], kind, p0, p1), gated_pair(ag[m][3], au[m][3], kind, p0, p1));
+      *reinterpret_cast<uint2*>(y + static_cast<size_t>(first + 16 * m + r) * ff + f0 + 4 * g) = make_uint2(o[0], o[1]);
+    }
+  }
+}
+
+template <int MT>
+__global__ __launch_bounds__(256) void moe_down_mfma_kernel(
+    const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
+    const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, int hidden, int ff,
+    float* __restrict__ rows) {
+  const int t = blockIdx.x;
+  if (t >= *n_tiles) return;
+  const int e = tiles[3 * t], first = tiles[3 * t + 1], count = tiles[3 * t + 2];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r = lane % 16, g = lane / 16;
+  const int h0 = (blockIdx.y * 4 + wave) * 16;
+  if (h0 >= hidden) return;
+  const bf16_t* wd = w + (static_cast<size_t>(e) * hidden + h0 + r) * ff + 8 * g;
+  const bf16_t* yr[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) yr[m] = y + static_cast<size_t>(first + min(16 * m + r, count - 1)) * ff + 8 * g;
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < ff; k0 += 32) {
+    MoeFrag a, b[MT];
+    a.u = *reinterpret_cast<const u32x4_t*>(wd + k0);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) b[m].u = *reinterpret_cast<const u32x4_t*>(yr[m] + k0);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[m].v, acc[m], 0, 0, 0);
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    if (16 * m + r < count) {
+      const int pair = order[first + 16 * m + r];
+      *reinterpret_cast<float4*>(rows + static_cast<size_t>(pair) * hidden + h0 + 4 * g) =
+          make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+    }
+  }
+}
+
+// Whether the matrix-core forms take these sizes (bfloat16 everywhere is the caller's to check).
+extern "C" int yk_moe_mfma_ok(int hidden, int ff, int x_stride) {
+  return hidden % 32 == 0 && ff % 32 == 0 && x_stride % 8 == 0;
+}
+
+static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+extern "C" int yk_moe_gate_up(const void* x, int x_stride, int dtype, const void* w, int w_dtype, const int32_t* order,
+                              const int32_t* slot_expert, const int32_t* tiles, const int32_t* n_tiles, int tile_rows,
+                              int max_tiles, int n_pairs, int top, int hidden, int ff, int kind, float p0, float p1,
+                              void* y, hipStream_t stream) {
+  YK_REQUIRE(n_pairs >= 0 && top >= 1 && hidden > 0 && ff > 0 && x_stride >= hidden, "moe_gate_up: bad sizes");
+  YK_REQUIRE(kind >= 0 && kind < YK_GATED_KINDS, "moe_gate_up: unknown activation");
+  if (n_pairs == 0) return 0;
+  if (dtype == YK_BF16 && w_dtype == YK_BF16 && yk_moe_mfma_ok(hidden, ff, x_stride) && aligned16(x) && aligned16(w) &&
+      aligned16(y) && (tile_rows == 16 || tile_rows == 64)) {
+    dim3 grid(max_tiles, (ff + 63) / 64), block(256);
+    if (tile_rows == 16)
+      moe_gate_up_mfma_kernel<1><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w),
+                                                            order, tiles, n_tiles, top, hidden, ff, kind, p0, p1, static_cast<bf16_t*>(y));
+    else
+      moe_gate_up_mfma_kernel<4><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w),
+                                                            order, tiles, n_tiles, top, hidden, ff, kind, p0, p1, static_cast<bf16_t*>(y));
+    return yk_check_launch("moe_gate_up (matrix cores)");
+  }
+  YK_REQUIRE(hidden <= 15 * 1024, "moe_gate_up: rows of more than 15,360 elements do not fit");
+  dim3 grid(n_pairs, std::min((ff + 255) / 256, 64)), block(256);
+  const size_t lds = static_cast<size_t>(hidden) * sizeof(float);
+#define YK_CASE(D, T, WD, TW)                                                                                     \
+  if (dtype == D && w_dtype == WD) {                                                                               \
+    moe_gate_up_fma_kernel<T, TW><<<grid, block, lds, stream>>>(static_cast<const T*>(x), x_stride, static_cast<const TW*>(w), \
+                                                                order, slot_expert, top, hidden, ff, kind, p0, p1,            \
+                                                                static_cast<T*>(y));                                          \
+    return yk_check_launch("moe_gate_up");                                                                         \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
+#undef YK_CASE
+  return yk_fail("moe_gate_up: unsupported dtype combination");
+}
+
+extern "C" int yk_moe_down(const void* y, int dtype, const void* w, int w_dtype, const int32_t* order,
+                           const int32_t* slot_expert, const int32_t* tiles, const int32_t* n_tiles, int tile_rows,
+                           int max_tiles, int n_pairs, int hidden, int ff, float* rows, hipStream_t stream) {
+  YK_REQUIRE(n_pairs >= 0 && hidden > 0 && ff > 0, "moe_down: bad sizes");
+  if (n_pairs == 0) return 0;
+  if (dtype == YK_BF16 && w_dtype == YK_BF16 && yk_moe_mfma_ok(ff, hidden, ff) && aligned16(y) && aligned16(w) &&
+      aligned16(rows) && (tile_rows == 16 || tile_rows == 64)) {
+    dim3 grid(max_tiles, (hidden + 63) / 64), block(256);
+    if (tile_rows == 16)
+      moe_down_mfma_kernel<1><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(y), static_cast<const bf16_t*>(w), order,
+                                                         tiles, n_tiles, hidden, ff, rows);
+    else
+      moe_down_mfma_kernel<4><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(y), static_cast<const bf16_t*>(w), order,
+                                                         tiles, n_tiles, hidden, ff, rows);
+    return yk_check_launch("moe_down (matrix cores)");
+  }
+  YK_REQUIRE(ff <= 15 * 1024, "moe_down: rows of more than 15,360 elements do not fit");
+  dim3 grid(n_pairs, std::min((hidden + 255) / 256, 64)), block(256);
+  const size_t lds = static_cast<size_t>(ff) * sizeof(float);
+#define YK_CASE(D, T, WD, TW)                                                                                    \
+  if (dtype == D && w_dtype == WD) {                                                                              \
+    moe_down_fma_kernel<T, TW><<<grid, block, lds, stream>>>(static_cast<const T*>(y), static_cast<const TW*>(w), order, \
+                                                             slot_expert, hidden, ff, rows);                            \
+    return yk_check_launch("moe_down");                                                                           \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
+#undef YK_CASE
+  return yk_fail("moe_down: unsupported dtype combination");
+}

@@ -131,7 +131,7 @@ class ModelRunner:
         self.rt = model.rt
         self.page_size = config.page_size
         n_pages = config.resolved_num_pages()
-        self.group_shapes = [GroupShape(n_pages, g.need.window) for g in model.cache_groups]
+        self.group_shapes = [GroupShape(n_pages, g.need.window, g.need.keep_first) for g in model.cache_groups]
         self.pages = PageManager(self.page_size, self.group_shapes, config.max_num_seqs)
         self.memory = CacheMemory(
             model,

@@ -59,7 +59,39 @@ _SIGNATURES = {
         _c_int,
     ),
     "yk_add_bias": ([_vp, _c_int, _c_int, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
-    "yk_gated_act": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_gated_act": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _vp], _c_int),
+    "yk_norm_add": (
+        [_vp, _vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _c_float, _vp, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_round_rows": ([_vp, _vp, _c_int, _c_size_t, _vp], _c_int),
+    "yk_qkv_prepare": (
+        [_vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int,
+         _c_int, _c_float, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _c_int,
+         _c_int, _vp],
+        _c_int,
+    ),
+    "yk_attn_masked": (
+        [_vp, _c_int, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+         _c_float, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_attn_finish": (
+        [_vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_causal_conv": ([_vp, _c_int, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_rglru_gates": ([_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_rglru_scan": ([_vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_moe_max_tiles": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_moe_mfma_ok": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_moe_route": ([_vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp], _c_int),
+    "yk_moe_gate_up": (
+        [_vp, _c_int, _c_int, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+         _c_float, _vp, _vp],
+        _c_int,
+    ),
+    "yk_moe_down": ([_vp, _c_int, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp], _c_int),
     "yk_gemm_fma": (
         [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
@@ -122,7 +154,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 16
+_ABI = 17
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -687,15 +719,16 @@ class HipOps:
         """act(x . gate^T) * (x . up^T) -> [M, intermediate], ``w_gate_up`` and ``group`` as
         ``pack_gate_up`` gave them.  Few rows of bfloat16 whose product is not split over K
         run as one kernel; otherwise the product, then the activation kernel."""
-        act = {"silu": 1, "gelu_tanh": 2}.get(activation)
+        act = {"silu": 1, "gelu_tanh": 2}.get(activation if isinstance(activation, str) else None)
         if act is None:
-            raise KernelError(f"unknown activation {activation!r}")
+            self.gated_kind(activation)  # raises for an unknown one
+            act = 0  # a gated pair that the product's epilogue does not have: product, then the activation kernel
         self._rows(x, "gate/up input")
         m, k = x.shape
         n = w_gate_up.shape[0]
         bf = torch.bfloat16
         fused = (
-            group == self.GATE_UP_GROUP and 0 < m <= SKINNY_MAX_ROWS and x.dtype == bf and w_gate_up.dtype == bf and out_dtype == bf
+            act > 0 and group == self.GATE_UP_GROUP and 0 < m <= SKINNY_MAX_ROWS and x.dtype == bf and w_gate_up.dtype == bf and out_dtype == bf
             and w_gate_up.shape[1] == k and k % 8 == 0 and x.stride(0) % 8 == 0 and w_gate_up.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0 and n % 16 == 0
             and self._ask("yk_gemm_skinny_splits", m, n, k, 1) == 1
@@ -945,9 +978,26 @@ class HipOps:
         return out
 
     # ----------------------------------------------------------------- activation
-    def gated_act(self, gu, activation: str, out_dtype: Optional[torch.dtype] = None, group: int = 0) -> torch.Tensor:
-        """act(gate) * up for gate/up columns [gate | up] (group 0) or alternating in groups
-        of ``group`` columns (see ``pack_gate_up``)."""
+    # gated pairs the kernels know: name -> (code, number of constants)
+    GATED_KINDS = {"silu": (0, 0), "gelu_tanh": (1, 0), "clamped_swish": (2, 2)}
+
+    @classmethod
+    def gated_kind(cls, activation) -> Tuple[int, float, float]:
+        """(code, p0, p1) of an activation given as a name or as (name, constants...):
+        ("clamped_swish", limit, slope) is min(g, limit) * sigmoid(slope * min(g, limit)) *
+        (clamp(u, -limit, limit) + 1)."""
+        name, consts = (activation, ()) if isinstance(activation, str) else (activation[0], tuple(activation[1:]))
+        if name not in cls.GATED_KINDS:
+            raise KernelError(f"unknown activation {name!r}")
+        code, n = cls.GATED_KINDS[name]
+        if len(consts) != n:
+            raise KernelError(f"activation {name!r} takes {n} constants, got {len(consts)}")
+        p = [float(c) for c in consts] + [0.0, 0.0]
+        return code, p[0], p[1]
+
+    def gated_act(self, gu, activation, out_dtype: Optional[torch.dtype] = None, group: int = 0) -> torch.Tensor:
+        """act(gate) * up (or another gated pair, see ``gated_kind``) for gate/up columns [gate | up]
+        (group 0) or alternating in groups of ``group`` columns (see ``pack_gate_up``)."""
         n_splits, round_sum = 1, 0
         src = gu
         if isinstance(gu, SplitSum):
@@ -963,16 +1013,288 @@ class HipOps:
             out_dtype = out_dtype or gu.dtype
         if cols % 2:
             raise KernelError("gate/up must have an even number of columns")
-        act = {"silu": 0, "gelu_tanh": 1}.get(activation)
-        if act is None:
-            raise KernelError(f"unknown activation {activation!r}")
+        act, p0, p1 = self.gated_kind(activation)
         inter = cols // 2
         out = torch.empty((rows, inter), dtype=out_dtype, device=src.device)
         self._check(
             self.lib.yk_gated_act(src.data_ptr(), _code(src.dtype), n_splits, round_sum, out.data_ptr(), _code(out_dtype),
-                                  rows, inter, act, int(group), self._stream())
+                                  rows, inter, act, int(group), p0, p1, self._stream())
         )
         return out
+
+    # ------------------------------------------------- a branch joins through its own norm
+    def round_rows(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        """A float32 stream rounded to the activation dtype (the stream itself when that is float32)."""
+        if out_dtype == torch.float32:
+            return x
+        if x.dtype != torch.float32 or not x.is_contiguous():
+            raise KernelError("round_rows takes a contiguous float32 tensor")
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        self._check(self.lib.yk_round_rows(x.data_ptr(), out.data_ptr(), _code(out_dtype), x.numel(), self._stream()))
+        return out
+
+    def norm_add(self, residual, branch, weight, eps, unit_offset, out_dtype, expert_rows=None, expert_weight: float = 1.0):
+        """residual (float32 [N, width], in place) += norm(branch) * weight, where branch is a tensor, a
+        ``SplitSum``, and / or ``expert_rows`` (float32 [N * top, width], of which a token takes
+        ``expert_weight`` times the sum of its top rows); returns the new residual in ``out_dtype``
+        (the residual itself for float32)."""
+        self._rows(residual, "residual")
+        if residual.dtype != torch.float32 or not residual.is_contiguous():
+            raise KernelError("the residual stream must be contiguous float32")
+        n, width = residual.shape
+        if weight.numel() != width:
+            raise KernelError(f"norm weight has {weight.numel()} elements, rows have {width}")
+        n_splits, round_sum, src = 1, 0, branch
+        if isinstance(branch, SplitAttention):
+            branch = src = branch.merge()
+        if isinstance(branch, SplitSum):
+            branch.check_live()
+            n_splits, round_sum, src = branch.n_splits, branch.round_sum, branch.tensor
+        if branch is not None and (tuple(branch.shape) != (n, width) or not src.is_contiguous()):
+            raise KernelError(f"branch {tuple(branch.shape)} does not match the residual {(n, width)}")
+        top = 0
+        if expert_rows is not None:
+            if expert_rows.dtype != torch.float32 or not expert_rows.is_contiguous() or expert_rows.dim() != 2 \
+                    or expert_rows.shape[1] != width or (n and expert_rows.shape[0] % n):
+                raise KernelError(f"expert rows {tuple(expert_rows.shape)} do not match the residual {(n, width)}")
+            top = expert_rows.shape[0] // n if n else 1
+        out = None if out_dtype == torch.float32 else torch.empty((n, width), dtype=out_dtype, device=residual.device)
+        self._check(
+            self.lib.yk_norm_add(
+                residual.data_ptr(), _ptr(src), 0 if src is None else _code(src.dtype), n_splits, round_sum,
+                _ptr(expert_rows), top, float(expert_weight), weight.data_ptr(), _code(weight.dtype), int(bool(unit_offset)),
+                float(eps), _ptr(out), _BF16, n, width, self._stream(),
+            )
+        )
+        return residual if out is None else out
+
+    # ------------------------------------- attention with prepared heads, kept first keys, a finish
+    def masked_pages_tiled(self, dtype: torch.dtype, head_dim: int, value_dim: int, page_size: int) -> bool:
+        return head_dim == value_dim and self.cache_tiled(dtype, head_dim, page_size)
+
+    def qkv_prepare(self, qkv, n_heads, n_kv, head_dim, value_dim, positions, act_dtype, q_norm=None, k_norm=None,
+                    qk_eps: float = 0.0, rotation=None, value_norm_eps=None, value_rotation=None,
+                    k_cache=None, v_cache=None, slots=None, page_size: int = 0) -> torch.Tensor:
+        """From a projection's rows [q | k | v | ...] (a tensor or a ``SplitSum``): normed (weights
+        ``q_norm`` / ``k_norm`` of head_dim elements, or none) and rotated queries [N, n_heads * head_dim];
+        normed, rotated keys and unit-normed (``value_norm_eps``), rotated (``value_rotation``) values
+        into the pages (``n_kv`` 0: queries only)."""
+        n_splits, round_sum, src = 1, 0, qkv
+        if isinstance(qkv, SplitSum):
+            qkv.check_live()
+            n_splits, round_sum, src = qkv.n_splits, qkv.round_sum, qkv.tensor
+            n, cols = qkv.shape
+            stride = cols
+        else:
+            self._rows(qkv, "qkv")
+            n, cols = qkv.shape
+            stride = qkv.stride(0)
+        if cols < n_heads * head_dim + n_kv * (head_dim + value_dim):
+            raise KernelError(f"qkv rows have {cols} elements, fewer than the heads need")
+        if positions.numel() != n or (n_kv > 0 and slots.numel() != n):
+            raise KernelError("positions/slots do not match the number of tokens")
+        q_out = torch.empty((n, n_heads * head_dim), dtype=act_dtype, device=src.device)
+        tiled = False
+        if n_kv > 0:
+            if k_cache.dtype != act_dtype or v_cache.dtype != act_dtype:
+                raise KernelError("cache and activations differ in dtype")
+            if tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or tuple(v_cache.shape[1:]) != (n_kv, value_dim, page_size):
+                raise KernelError(f"cache pages have shapes {tuple(k_cache.shape)}, {tuple(v_cache.shape)}")
+            tiled = self.masked_pages_tiled(act_dtype, head_dim, value_dim, page_size)
+        norm_w = q_norm if q_norm is not None else k_norm
+        if q_norm is not None and k_norm is not None and q_norm.dtype != k_norm.dtype:
+            raise KernelError("query and key norm weights differ in dtype")
+        for w in (q_norm, k_norm):
+            if w is not None and (w.numel() != head_dim or not w.is_contiguous()):
+                raise KernelError(f"a head norm's weight has {w.numel()} elements, heads have {head_dim}")
+        qk_norm = int(q_norm is not None or k_norm is not None)
+        if qk_norm and (q_norm is None or k_norm is None):
+            raise KernelError("queries and keys are normed together or not at all")
+        for r in (rotation, value_rotation):
+            if r is not None and (r.cos.dtype != torch.float32 or r.cos.shape != r.sin.shape or r.cos.shape[1] != r.rotary_dim // 2):
+                raise KernelError("rotary tables must be float32 [positions, rotary_dim/2]")
+        if value_rotation is not None and value_rotation.rotary_dim != value_dim:
+            raise KernelError("values rotate over all of value_dim")
+        self._check(
+            self.lib.yk_qkv_prepare(
+                src.data_ptr(), _code(src.dtype), n_splits, round_sum, stride, q_out.data_ptr(), _code(act_dtype),
+                q_out.stride(0), n, n_heads, n_kv, head_dim, value_dim, positions.data_ptr(), _ptr(q_norm), _ptr(k_norm),
+                _F32 if norm_w is None else _code(norm_w.dtype), qk_norm, float(qk_eps),
+                None if rotation is None else rotation.cos.data_ptr(), None if rotation is None else rotation.sin.data_ptr(),
+                0 if rotation is None else rotation.rotary_dim, int(bool(rotation is not None and rotation.interleaved)),
+                0 if rotation is None else rotation.cos.shape[0],
+                int(value_norm_eps is not None), float(value_norm_eps or 0.0),
+                None if value_rotation is None else value_rotation.cos.data_ptr(),
+                None if value_rotation is None else value_rotation.sin.data_ptr(),
+                int(bool(value_rotation is not None and value_rotation.interleaved)),
+                0 if value_rotation is None else value_rotation.cos.shape[0],
+                _ptr(k_cache) if n_kv else None, _ptr(v_cache) if n_kv else None, _ptr(slots) if n_kv else None,
+                int(page_size), int(tiled), self._stream(),
+            )
+        )
+        return q_out
+
+    @staticmethod
+    def _gate_source(gate, n: int):
+        """(tensor, splits, round_sum, row stride) of the projection whose columns hold per-head gates."""
+        if gate is None:
+            return None, 1, 0, 0
+        if isinstance(gate, SplitSum):
+            gate.check_live()
+            return gate.tensor, gate.n_splits, gate.round_sum, gate.shape[1]
+        return gate, 1, 0, gate.stride(0)
+
+    def attention_masked(self, q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, page_size, scale, ctx, group,
+                         window: int = 0, keep_first: int = 0, softcap: float = 0.0, value_rotation=None,
+                         gate=None, gate_col: int = 0) -> torch.Tensor:
+        """softmax over the keys j <= p with (p - j < window or j < keep_first) of q . k * scale
+        (squashed by ``softcap`` * tanh(s / ``softcap``) when set), times the values [N, n_heads *
+        value_dim]; then, with ``value_rotation``, every head's output turned back by its token's
+        position, and, with ``gate`` (the projection, a tensor or ``SplitSum``, whose columns
+        ``gate_col`` + h hold the heads' gates), multiplied by the sigmoid of its gate."""
+        self._rows(q, "queries")
+        n = q.shape[0]
+        bt = ctx.arrays[f"block_table_g{group}"]
+        if tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or tuple(v_cache.shape[1:]) != (n_kv, value_dim, page_size):
+            raise KernelError(f"cache pages have shapes {tuple(k_cache.shape)}, {tuple(v_cache.shape)}")
+        if k_cache.dtype != q.dtype:
+            raise KernelError("cache and activations differ in dtype")
+        out = torch.empty((n, n_heads * value_dim), dtype=q.dtype, device=q.device)
+        gsrc, gsplits, ground, gstride = self._gate_source(gate, n)
+        vr = value_rotation
+        self._check(
+            self.lib.yk_attn_masked(
+                q.data_ptr(), q.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype),
+                ctx.arrays["positions"].data_ptr(), ctx.arrays["token_seq"].data_ptr(), bt.data_ptr(), bt.shape[1], n,
+                page_size, head_dim, value_dim, n_heads, n_kv, float(scale), float(softcap or 0.0), int(window or 0),
+                int(keep_first or 0), int(self.masked_pages_tiled(q.dtype, head_dim, value_dim, page_size)),
+                None if vr is None else vr.cos.data_ptr(), None if vr is None else vr.sin.data_ptr(),
+                int(bool(vr is not None and vr.interleaved)), 0 if vr is None else vr.cos.shape[0],
+                _ptr(gsrc), 0 if gsrc is None else _code(gsrc.dtype), gsplits, ground, gstride, int(gate_col), self._stream(),
+            )
+        )
+        return out
+
+    def attention_finish(self, out, positions, n_heads, value_dim, value_rotation=None, gate=None, gate_col: int = 0):
+        """In place on an attention's output [N, n_heads * value_dim]: the turn back by the position
+        and the gate, as ``attention_masked`` applies them itself."""
+        n = out.shape[0]
+        gsrc, gsplits, ground, gstride = self._gate_source(gate, n)
+        vr = value_rotation
+        self._check(
+            self.lib.yk_attn_finish(
+                out.data_ptr(), _code(out.dtype), positions.data_ptr(), n, value_dim, n_heads,
+                None if vr is None else vr.cos.data_ptr(), None if vr is None else vr.sin.data_ptr(),
+                int(bool(vr is not None and vr.interleaved)), 0 if vr is None else vr.cos.shape[0],
+                _ptr(gsrc), 0 if gsrc is None else _code(gsrc.dtype), gsplits, ground, gstride, int(gate_col), self._stream(),
+            )
+        )
+        return out
+
+    # ------------------------------------------------ short convolution + gated linear recurrence
+    def causal_conv(self, x, weight, bias, state, ctx) -> torch.Tensor:
+        """Per channel, u_t = bias + sum_j weight[c, j] * x_(t - (taps - 1 - j)) over each request's
+        span; inputs before the span come from ``state`` [slots, taps - 1, channels] (not changed here).
+        ``x`` [N, channels] may be a view with a row stride."""
+        n, channels = x.shape
+        taps = weight.shape[1]
+        if x.stride(1) != 1 or tuple(weight.shape) != (channels, taps) or not weight.is_contiguous():
+            raise KernelError("causal_conv: x must have unit column stride and weight be [channels, taps]")
+        if bias is not None and (bias.dtype != weight.dtype or bias.numel() != channels):
+            raise KernelError("causal_conv: bias does not match the weight")
+        if taps > 1 and (state.dtype != x.dtype or tuple(state.shape[1:]) != (taps - 1, channels)):
+            raise KernelError(f"causal_conv: state {tuple(state.shape)} does not hold {taps - 1} inputs of {channels} channels")
+        out = torch.empty((n, channels), dtype=x.dtype, device=x.device)
+        a = ctx.arrays
+        self._check(
+            self.lib.yk_causal_conv(
+                x.data_ptr(), x.stride(0), _code(x.dtype), weight.data_ptr(), _ptr(bias), _code(weight.dtype), _ptr(state),
+                a["token_seq"].data_ptr(), a["seq_qstart"].data_ptr(), a["state_slots"].data_ptr(), out.data_ptr(),
+                n, channels, taps, self._stream(),
+            )
+        )
+        return out
+
+    def rglru(self, u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx) -> torch.Tensor:
+        """The real-gated linear recurrence over each request's span.  ``u`` [N, C] the convolved
+        branch, ``y`` [N, C] the other branch before its gelu, ``x`` [N, C] the convolution's inputs (its
+        state is brought up to date here); gate matrices transposed [blocks, in, out].  Returns S_t *
+        gelu(y_t) [N, C]; ``s_state`` [slots, C] float32 and ``conv_state`` are left as after the span."""
+        n, channels = u.shape
+        blocks = wa_t.shape[0]
+        bs = channels // blocks
+        if tuple(wa_t.shape) != (blocks, bs, bs) or tuple(wi_t.shape) != (blocks, bs, bs) or not wa_t.is_contiguous() or not wi_t.is_contiguous():
+            raise KernelError("rglru: gate matrices must be contiguous [blocks, width / blocks, width / blocks]")
+        for t in (ba, bi, lam):
+            if t.numel() != channels or t.dtype != wa_t.dtype or not t.is_contiguous():
+                raise KernelError("rglru: gate biases and decay parameters are [width] in the matrices' dtype")
+        if s_state.dtype != torch.float32 or s_state.shape[1] != channels:
+            raise KernelError("rglru: the recurrent state is float32 [slots, width]")
+        if not u.is_contiguous() or y.stride(1) != 1 or x.stride(1) != 1 or y.dtype != u.dtype or x.dtype != u.dtype:
+            raise KernelError("rglru: branches must share a dtype and have unit column stride")
+        a = torch.empty((n, channels), dtype=torch.float32, device=u.device)
+        b = torch.empty((n, channels), dtype=torch.float32, device=u.device)
+        self._check(
+            self.lib.yk_rglru_gates(
+                u.data_ptr(), _code(u.dtype), wa_t.data_ptr(), ba.data_ptr(), wi_t.data_ptr(), bi.data_ptr(), lam.data_ptr(),
+                _code(wa_t.dtype), float(rate), a.data_ptr(), b.data_ptr(), n, channels, blocks, self._stream(),
+            )
+        )
+        out = torch.empty((n, channels), dtype=u.dtype, device=u.device)
+        arr = ctx.arrays
+        self._check(
+            self.lib.yk_rglru_scan(
+                a.data_ptr(), b.data_ptr(), y.data_ptr(), y.stride(0), x.data_ptr(), x.stride(0), _code(u.dtype),
+                s_state.data_ptr(), _ptr(conv_state), arr["seq_qstart"].data_ptr(), arr["seq_qlen"].data_ptr(),
+                arr["state_slots"].data_ptr(), out.data_ptr(), arr["seq_qstart"].numel(), channels, int(taps), self._stream(),
+            )
+        )
+        return out
+
+    # --------------------------------------------------------------- mixture of experts
+    def moe_experts(self, x, token_ids, table, w_gate_up, w_down, activation) -> torch.Tensor:
+        """Every token through the experts its id names in ``table`` [vocab, top]: returns float32
+        rows [N * top, hidden], row n * top + k the output of token n's k-th expert (uncombined).
+        ``w_gate_up`` [experts, 2, ff, hidden] (gate rows, then up rows), ``w_down`` [experts, hidden, ff]."""
+        self._rows(x, "expert input")
+        n, hidden = x.shape
+        vocab, top = table.shape
+        experts, two, ff, hid = w_gate_up.shape
+        if two != 2 or hid != hidden or tuple(w_down.shape) != (experts, hidden, ff) or not w_gate_up.is_contiguous() or not w_down.is_contiguous():
+            raise KernelError("moe: expert weights must be contiguous [experts, 2, ff, hidden] and [experts, hidden, ff]")
+        if table.dtype != torch.int32 or not table.is_contiguous() or token_ids.dtype != torch.int32 or token_ids.numel() != n:
+            raise KernelError("moe: the table and the token ids are int32, one id per row")
+        kind, p0, p1 = self.gated_kind(activation)
+        pairs = n * top
+        dev = x.device
+        rows = torch.empty((pairs, hidden), dtype=torch.float32, device=dev)
+        if n == 0:
+            return rows
+        # tiles of 64 pairs where an expert has that many on average, else of 16
+        tile_rows = 64 if pairs >= 48 * experts else 16
+        max_tiles = self.lib.yk_moe_max_tiles(pairs, experts, tile_rows)
+        ints = torch.empty(2 * pairs + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
+        order, slot_expert = ints[:pairs], ints[pairs: 2 * pairs]
+        tiles, n_tiles = ints[2 * pairs: 2 * pairs + 3 * max_tiles], ints[2 * pairs + 3 * max_tiles:]
+        self._check(
+            self.lib.yk_moe_route(token_ids.data_ptr(), table.data_ptr(), vocab, top, experts, n, tile_rows, order.data_ptr(),
+                                  slot_expert.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), self._stream())
+        )
+        y = torch.empty((pairs, ff), dtype=x.dtype, device=dev)
+        self._check(
+            self.lib.yk_moe_gate_up(
+                x.data_ptr(), x.stride(0), _code(x.dtype), w_gate_up.data_ptr(), _code(w_gate_up.dtype), order.data_ptr(),
+                slot_expert.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), tile_rows, max_tiles, pairs, top, hidden, ff,
+                kind, p0, p1, y.data_ptr(), self._stream(),
+            )
+        )
+        self._check(
+            self.lib.yk_moe_down(
+                y.data_ptr(), _code(y.dtype), w_down.data_ptr(), _code(w_down.dtype), order.data_ptr(), slot_expert.data_ptr(),
+                tiles.data_ptr(), n_tiles.data_ptr(), tile_rows, max_tiles, pairs, hidden, ff, rows.data_ptr(), self._stream(),
+            )
+        )
+        return rows
 
     # ------------------------------------------------------------------- sampling
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:

@@ -13,6 +13,18 @@ params: prefix, hidden_size, num_heads, num_kv_heads, head_dim, scale, window
 encoding's ``rotation()``), names (optional overrides of the tensor names below the
 prefix), bias (False; True: the four projections have biases ``*.bias`` beside their
 weights, which Llama's do not).
+
+Options beyond the plain causal form (any of them sends the layer through the kernels that
+prepare, mask and finish heads in general, ``ops.qkv_prepare`` / ``ops.attention_masked``):
+value_dim (values narrower or wider than keys), qk_norm ({"q": name, "k": name, "eps": e}: an RMS
+norm per head on queries and keys before the rotation, its weight of head_dim elements shared by
+the heads), value_norm_eps (values divided by their root mean square per head before they are
+cached), value_position (a rotary PartSpec over all of value_dim: values are cached rotated by
+their position and a head's output is turned back by the query's position, so that what reaches
+the output depends on distances), softcap (scores squashed to softcap * tanh(s / softcap)),
+keep_first (that many first keys stay visible below the window), gate (a tensor name below the
+prefix, [num_heads, hidden]: a head's output is multiplied by the sigmoid of its row's product with
+the mixer's input).
 """
 from __future__ import annotations
 
@@ -56,6 +68,30 @@ class Attention(Mixer):
             raise ValueError(f"{self.prefix}: position encoding {pos.kind!r} offers no rotation, which is all this mixer applies")
         if self.rotation is not None and self.rotation.rotary_dim > self.head_dim:
             raise ValueError("rotary_dim exceeds head_dim")
+        self.value_dim = int(params.get("value_dim") or self.head_dim)
+        self.qk_norm = params.get("qk_norm")
+        self.value_norm_eps = params.get("value_norm_eps")
+        vpos: PartSpec = params.get("value_position")
+        self.value_position = None if vpos is None else POSITIONS.get(vpos.kind)(vpos.params, rt)
+        self.value_rotation = None if self.value_position is None else self.value_position.rotation()
+        if self.value_rotation is not None and self.value_rotation.rotary_dim != self.value_dim:
+            raise ValueError(f"{self.prefix}: values rotate over all of value_dim={self.value_dim}")
+        self.softcap = float(params.get("softcap") or 0.0)
+        self.keep_first = int(params.get("keep_first") or 0)
+        self.gate_name = params.get("gate")
+        self.masked = bool(
+            self.value_dim != self.head_dim or self.qk_norm or self.value_norm_eps is not None or self.value_rotation is not None
+            or self.softcap or self.keep_first or self.gate_name
+        )
+        self.w_qn = self.w_kn = None
+        if self.masked:
+            if self.bias:
+                raise ValueError(f"{self.prefix}: biases are not offered together with the masked attention's options")
+            self.group = None
+            self.w_qkv = self.w_q = self.w_o = None
+            self.b_qkv = self.b_q = self.b_o = None
+            self.rotates_in_launch = False
+            return
         rt.ops.check_attention_sizes(self.n_heads, self.n_kv, self.head_dim, rt.page_size)
         self.tokens_per_tile = rt.ops.attention_tokens_per_tile(self.n_heads, self.n_kv)
         # spans longer than `long_tile` go to the kernel for long spans, in tiles of that many
@@ -79,11 +115,17 @@ class Attention(Mixer):
         kd = self.n_kv * self.head_dim
         specs = {
             self.names["q"]: TensorSpec((hd, self.hidden)),
-            self.names["o"]: TensorSpec((self.hidden, hd)),
+            self.names["o"]: TensorSpec((self.hidden, self.n_heads * self.value_dim)),
         }
         if self.projects_kv:
             specs[self.names["k"]] = TensorSpec((kd, self.hidden))
-            specs[self.names["v"]] = TensorSpec((kd, self.hidden))
+            specs[self.names["v"]] = TensorSpec((self.n_kv * self.value_dim, self.hidden))
+        if self.qk_norm:
+            specs[f"{self.prefix}.{self.qk_norm['q']}"] = TensorSpec((self.head_dim,), "float", ("one_plus_normal", 0.1))
+            if self.projects_kv:
+                specs[f"{self.prefix}.{self.qk_norm['k']}"] = TensorSpec((self.head_dim,), "float", ("one_plus_normal", 0.1))
+        if self.gate_name:
+            specs[f"{self.prefix}.{self.gate_name}"] = TensorSpec((self.n_heads, self.hidden))
         if self.bias:
             for which, spec in list(specs.items()):
                 specs[self._bias_name(which)] = TensorSpec((spec.shape[0],), "float", ("normal", 0.02))
@@ -95,6 +137,24 @@ class Attention(Mixer):
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         q = tensors[self.names["q"]]
+        if self.masked:
+            # one projection for everything that reads the mixer's input: [q; k; v; gates], its rows
+            # padded to a multiple of 8 so that the few-row product's tiles take it
+            parts = [q]
+            if self.projects_kv:
+                parts += [tensors[self.names["k"]], tensors[self.names["v"]]]
+            if self.gate_name:
+                parts.append(tensors[f"{self.prefix}.{self.gate_name}"])
+            rows = sum(p.shape[0] for p in parts)
+            pad = -rows % 16
+            if pad:
+                parts.append(torch.zeros((pad, self.hidden), dtype=q.dtype, device=q.device))
+            self.w_qkv = torch.cat(parts, dim=0).contiguous()
+            self.w_o = tensors[self.names["o"]]
+            if self.qk_norm:
+                self.w_qn = tensors[f"{self.prefix}.{self.qk_norm['q']}"]
+                self.w_kn = tensors[f"{self.prefix}.{self.qk_norm['k']}"] if self.projects_kv else self.w_qn
+            return
         if self.projects_kv:
             self.w_qkv = torch.cat([q, tensors[self.names["k"]], tensors[self.names["v"]]], dim=0).contiguous()
             self.w_q = self.w_qkv[: q.shape[0]]
@@ -111,10 +171,14 @@ class Attention(Mixer):
             self.b_o = b("o")
 
     def kv_need(self) -> KVNeed:
-        return KVNeed(self.n_kv, self.head_dim, self.window)
+        return KVNeed(self.n_kv, self.head_dim, self.window, None if self.value_dim == self.head_dim else self.value_dim,
+                      self.keep_first if self.window else 0)
 
     def products(self):
         hd, kd = self.n_heads * self.head_dim, self.n_kv * self.head_dim
+        if self.masked:
+            rows = hd + (kd + self.n_kv * self.value_dim if self.projects_kv else 0) + (self.n_heads if self.gate_name else 0)
+            return ((rows + (-rows % 16), self.hidden), (self.hidden, self.n_heads * self.value_dim))
         return ((hd + 2 * kd if self.projects_kv else hd, self.hidden), (self.hidden, hd))
 
     def long_col_tiles(self, hb) -> int:
@@ -132,6 +196,8 @@ class Attention(Mixer):
         return self.rt.ops.attention_long_col_tiles(tiles * self.n_kv * chunks, fewest)
 
     def step_inputs(self):
+        if self.masked:
+            return {}
         # spans of more than one large tile go to the kernel for long spans, the rest
         # (single decoded tokens, short portions) to the one that splits the keys
         tpt = self.tokens_per_tile
@@ -149,7 +215,31 @@ class Attention(Mixer):
         }
 
     # ---- what it computes
+    def _forward_masked(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
+        ops = self.rt.ops
+        if site.owns_cache != self.projects_kv:
+            raise RuntimeError(f"{self.prefix}: a layer whose run entries both own and borrow caches is not offered with these options")
+        proj = ops.linear(h, self.w_qkv, self.rt.act_dtype, partial_ok=True)
+        n_kv_rows = self.n_kv if site.owns_cache else 0
+        k_cache, v_cache = site.kv()
+        q = ops.qkv_prepare(
+            proj, self.n_heads, n_kv_rows, self.head_dim, self.value_dim, ctx.arrays["positions"], self.rt.act_dtype,
+            q_norm=self.w_qn, k_norm=self.w_kn, qk_eps=float(self.qk_norm["eps"]) if self.qk_norm else 0.0,
+            rotation=self.rotation, value_norm_eps=self.value_norm_eps, value_rotation=self.value_rotation,
+            k_cache=k_cache, v_cache=v_cache, slots=ctx.arrays[f"slots_g{site.group}"] if n_kv_rows else None,
+            page_size=self.rt.page_size,
+        )
+        gate_col = self.n_heads * self.head_dim + n_kv_rows * (self.head_dim + self.value_dim)
+        out = ops.attention_masked(
+            q, self.n_heads, self.n_kv, self.head_dim, self.value_dim, k_cache, v_cache, self.rt.page_size, self.scale, ctx,
+            site.group, window=0 if self.window is None else int(self.window), keep_first=self.keep_first,
+            softcap=self.softcap, value_rotation=self.value_rotation, gate=proj if self.gate_name else None, gate_col=gate_col,
+        )
+        return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
+
     def forward(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
+        if self.masked:
+            return self._forward_masked(h, ctx, site)
         ops = self.rt.ops
         if site.owns_cache:
             if not self.projects_kv:

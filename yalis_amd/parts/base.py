@@ -38,12 +38,15 @@ class KVNeed:
     """A mixer's need for cached keys and values: per token ``num_kv_heads`` rows
     of ``head_dim`` for keys and of ``value_dim`` for values (None: as wide as the keys;
     0: no values are kept, the pages hold keys only, e.g. one compressed row per token).
-    ``window`` = how many of the latest tokens are ever read again (None: all of them)."""
+    ``window`` = how many of the latest tokens are ever read again (None: all of them);
+    ``keep_first`` = how many of the first tokens stay readable whatever the window says (their
+    pages are never given back while the request lives)."""
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
+    keep_first: int = 0
 
     @property
     def v_dim(self) -> int:
@@ -70,6 +73,17 @@ class Rotation:
     sin: torch.Tensor
     rotary_dim: int
     interleaved: bool = False
+
+
+class Settled:
+    """What a block hands on in place of a pending contribution when it has added everything to
+    the residual itself: nothing is left to add, and ``activations`` is the residual stream as
+    it now stands in the activation dtype (the residual itself in the float32 engine), which a
+    block whose branches read the stream un-normed would otherwise have to make again.  Norms
+    treat it as "nothing to add"."""
+
+    def __init__(self, activations: torch.Tensor):
+        self.activations = activations
 
 
 class Part:
@@ -130,6 +144,26 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class ExpertRows:
+    """A feed-forward's output not yet summed: ``dense`` (a tensor, a product's unreduced slices,
+    or None) plus ``weight`` times the sum of each token's ``top`` consecutive rows of ``rows``
+    (float32 [tokens * top, width]).  A norm's ``norm_add`` sums them while it reads them;
+    ``combine()`` gives the tensor for whoever cannot."""
+
+    def __init__(self, dense, rows: torch.Tensor, top: int, weight: float):
+        self.dense, self.rows, self.top, self.weight = dense, rows, int(top), float(weight)
+        self.shape = (rows.shape[0] // self.top, rows.shape[1])
+
+    def combine(self) -> torch.Tensor:
+        out = self.rows.view(self.shape[0], self.top, self.shape[1]).sum(1) * self.weight
+        if self.dense is not None:
+            out = out + self.dense.float()
+        return out
+
+    def float(self) -> torch.Tensor:
+        return self.combine()
+
+
 class Norm(Part):
     # True when ``add_norm`` hands ``delta`` to a kernel library that understands an embedding's
     # ungathered rows (``ops.embedded_rows``) in its place
@@ -148,6 +182,13 @@ class Norm(Part):
 
     def gather_add_norm(self, residual, delta, rows) -> torch.Tensor:
         """The same on the rows ``rows`` only, without changing ``residual``."""
+        raise NotImplementedError
+
+    def norm_add(self, residual: torch.Tensor, branch, expert_rows=None, expert_weight: float = 1.0) -> torch.Tensor:
+        """residual (float32, in place) += norm(branch): a branch's output is normed on its way into
+        the stream.  ``branch`` is whatever a part's ``forward`` returned, and / or the uncombined rows
+        of a mixture of experts (``FeedForward.forward`` may return an ``ExpertRows``).  Returns the
+        new residual in the activation dtype."""
         raise NotImplementedError
 
 

@@ -11,7 +11,7 @@ returns its own last contribution, to be added by whoever comes next.
 """
 from __future__ import annotations
 
-from .base import Block, register_block
+from .base import Block, Settled, register_block
 
 
 @register_block("prenorm")
@@ -38,3 +38,41 @@ class PreNormBlock(Block):
         a = self.mixer.forward(h, ctx, site)
         h = self.feed_forward_norm.add_norm(residual, a)
         return self.feed_forward.forward(h, ctx)
+
+
+@register_block("branch_norm")
+class BranchNormBlock(Block):
+    """Norms on the branches' outputs only: x = x + norm_1(mixer(x)); x = x + norm_2(feed_forward(x)).
+    The branches read the stream itself.  A layer may leave the feed-forward (and its norm) out.
+
+    Every addition happens inside the block (a pending contribution would have to wait for a norm
+    that is not there), so what it hands on is ``Settled``: the stream in the activation dtype,
+    which the norm's kernel writes beside the float32 residual in the same pass, and which the next
+    block of this kind reads instead of rounding the residual again."""
+
+    roles = {
+        "mixer": ("mixer", True),
+        "mixer_norm": ("norm", True),
+        "feed_forward": ("feed_forward", False),
+        "feed_forward_norm": ("norm", False),
+    }
+
+    def __init__(self, mixer, mixer_norm, feed_forward=None, feed_forward_norm=None):
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("a branch_norm block has a feed-forward and its norm, or neither")
+        self.mixer = mixer
+        self.mixer_norm = mixer_norm
+        self.feed_forward = feed_forward
+        self.feed_forward_norm = feed_forward_norm
+
+    def forward(self, residual, delta, ctx, site):
+        if isinstance(delta, Settled):
+            h = delta.activations
+        else:
+            if delta is not None:  # a block of another kind left a contribution: it is added as it is
+                residual += delta.float()
+            h = self.mixer.rt.ops.round_rows(residual, self.mixer.rt.act_dtype)
+        h = self.mixer_norm.norm_add(residual, self.mixer.forward(h, ctx, site))
+        if self.feed_forward is not None:
+            h = self.feed_forward_norm.norm_add(residual, self.feed_forward.forward(h, ctx))
+        return Settled(h)

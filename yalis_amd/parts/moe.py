@@ -1,0 +1,102 @@
+"""A mixture of small gated feed-forward experts whose choice is a table over token ids.
+
+Every token id has ``top`` experts of ``experts`` (a row of the integer table [vocab, top], its
+entries distinct); the token's output is the mean of theirs (each weighs 1 / top).  No router is
+computed: the experts of a token follow from the token alone, so the routing of a step is known
+from its token ids (on the device: a step may take its tokens from what the step before sampled).
+An optional shared expert of its own width runs for every token and is added.
+
+An expert is a gated feed-forward without biases whose activation is a parameter
+(``ops.gated_kind``); the design that brought it uses ("clamped_swish", limit, slope).
+
+What ``forward`` returns is an ``ExpertRows``: the shared expert's output (possibly still the
+unreduced slices of its down projection) beside the experts' uncombined rows; the norm that takes
+the branch into the residual adds them while it reads them.
+
+params: prefix, hidden_size, vocab_size, experts, top, intermediate_size, activation, shared
+(None or {"intermediate_size", "activation"}), names (optional: "table", "expert" with {e} for
+the expert's number, "shared", "gate", "up", "down").
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping
+
+import torch
+
+from ..weights.loader import TensorSpec
+from .base import ExpertRows, FeedForward, Runtime, register_feed_forward
+
+
+@register_feed_forward("table_moe")
+class TableMoE(FeedForward):
+    graph_capturable = True
+
+    def __init__(self, params, rt: Runtime):
+        super().__init__(params, rt)
+        self.prefix = params["prefix"]
+        self.hidden = int(params["hidden_size"])
+        self.vocab = int(params["vocab_size"])
+        self.experts = int(params["experts"])
+        self.top = int(params["top"])
+        self.inter = int(params["intermediate_size"])
+        self.activation = params.get("activation", "silu")
+        if not 1 <= self.top <= self.experts:
+            raise ValueError(f"{self.prefix}: top={self.top} of {self.experts} experts")
+        rt.ops.gated_kind(self.activation)  # raises for one the kernels do not know
+        self.shared = params.get("shared")
+        names = {"table": "table", "expert": "e{e}", "shared": "shared", "gate": "gate", "up": "up", "down": "down"}
+        names.update(params.get("names", {}))
+        self.names = names
+        self.table = self.w_gate_up = self.w_down = None
+        self.shared_gate_up = self.shared_down = None
+        self.shared_group = 0
+
+    def _name(self, owner: str, which: str) -> str:
+        return f"{self.prefix}.{owner}.{self.names[which]}"
+
+    def _expert(self, e: int) -> str:
+        return self.names["expert"].format(e=e)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = {f"{self.prefix}.{self.names['table']}": TensorSpec((self.vocab, self.top), "int", ("distinct", self.experts))}
+        for e in range(self.experts):
+            specs[self._name(self._expert(e), "gate")] = TensorSpec((self.inter, self.hidden))
+            specs[self._name(self._expert(e), "up")] = TensorSpec((self.inter, self.hidden))
+            specs[self._name(self._expert(e), "down")] = TensorSpec((self.hidden, self.inter))
+        if self.shared:
+            ff = int(self.shared["intermediate_size"])
+            specs[self._name(self.names["shared"], "gate")] = TensorSpec((ff, self.hidden))
+            specs[self._name(self.names["shared"], "up")] = TensorSpec((ff, self.hidden))
+            specs[self._name(self.names["shared"], "down")] = TensorSpec((self.hidden, ff))
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        table = tensors[f"{self.prefix}.{self.names['table']}"]
+        if int(table.min()) < 0 or int(table.max()) >= self.experts:
+            raise ValueError(f"{self.prefix}: the table names experts outside 0..{self.experts - 1}")
+        self.table = table.to(torch.int32).contiguous()
+        # all experts in two tensors: [experts, 2, ff, hidden] (gate rows, then up rows) and [experts, hidden, ff]
+        self.w_gate_up = torch.stack([
+            torch.stack([tensors[self._name(self._expert(e), "gate")], tensors[self._name(self._expert(e), "up")]])
+            for e in range(self.experts)
+        ]).contiguous()
+        self.w_down = torch.stack([tensors[self._name(self._expert(e), "down")] for e in range(self.experts)]).contiguous()
+        if self.shared:
+            s = self.names["shared"]
+            self.shared_gate_up, self.shared_group = self.rt.ops.pack_gate_up(tensors[self._name(s, "gate")], tensors[self._name(s, "up")])
+            self.shared_down = tensors[self._name(s, "down")]
+
+    def products(self):
+        if not self.shared:
+            return ()
+        ff = int(self.shared["intermediate_size"])
+        return ((2 * ff, self.hidden), (self.hidden, ff))
+
+    def forward(self, h: torch.Tensor, ctx):
+        ops = self.rt.ops
+        rows = ops.moe_experts(h, ctx.arrays["token_ids"], self.table, self.w_gate_up, self.w_down, self.activation)
+        dense = None
+        if self.shared:
+            a = ops.gate_up_act(h, self.shared_gate_up, self.shared_group, self.shared["activation"], self.rt.act_dtype)
+            dense = ops.linear(a, self.shared_down, self.rt.act_dtype, partial_ok=True)
+        return ExpertRows(dense, rows, self.top, 1.0 / self.top)

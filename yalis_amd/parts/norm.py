@@ -4,7 +4,8 @@ out = x * rsqrt(mean(x^2) + eps) * weight, all in float32 with one rounding at
 the end; ``unit_offset`` multiplies by (1 + weight) instead (a flag of the same
 class in the reference, :984).  The kernel fuses the residual sum that precedes
 every norm of a pre-norm block: the float32 residual stream is updated in place
-and normalised in one pass.
+and normalised in one pass.  ``norm_add`` is the other way round, for blocks that norm a
+branch's output instead of its input: residual += norm(branch), again one pass.
 """
 from __future__ import annotations
 
@@ -13,7 +14,7 @@ from typing import Dict, Mapping, Optional
 import torch
 
 from ..weights.loader import TensorSpec
-from .base import Norm, Runtime, register_norm
+from .base import ExpertRows, Norm, Runtime, Settled, register_norm
 
 
 @register_norm("rmsnorm")
@@ -41,11 +42,21 @@ class RMSNorm(Norm):
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.unit_offset, self.rt.act_dtype)
 
     def add_norm(self, residual, delta):
+        if isinstance(delta, Settled):
+            delta = None
         return self.rt.ops.add_rmsnorm(
             residual, delta, self.weight, self.eps, self.unit_offset, self.rt.act_dtype
         )
 
+    def norm_add(self, residual, branch, expert_rows=None, expert_weight=1.0):
+        if isinstance(branch, ExpertRows):
+            branch, expert_rows, expert_weight = branch.dense, branch.rows, branch.weight
+        return self.rt.ops.norm_add(residual, branch, self.weight, self.eps, self.unit_offset, self.rt.act_dtype,
+                                    expert_rows=expert_rows, expert_weight=expert_weight)
+
     def gather_add_norm(self, residual, delta, rows):
+        if isinstance(delta, Settled):
+            delta = None
         return self.rt.ops.gather_add_rmsnorm(
             residual, delta, rows, self.weight, self.eps, self.unit_offset, self.rt.act_dtype
         )

@@ -8,8 +8,14 @@ in the kernel that also appends keys and values to the cache.
 
 params: rotary_dim (how many leading elements of each head rotate), theta,
 pairing ("half": (i, i + rotary_dim/2); "interleaved": (2i, 2i+1)),
-scaling (None or {"kind": "llama3", factor, low_freq_factor, high_freq_factor,
-original_max_position_embeddings}).
+scaling (None, {"kind": "llama3", factor, low_freq_factor, high_freq_factor,
+original_max_position_embeddings}, or {"kind": "yarn", factor, original, fast, slow}).
+
+"yarn" (Peng et al., "YaRN: Efficient Context Window Extension of Large Language Models"): pairs
+whose wavelength is short against the original context keep their frequency, pairs whose
+wavelength is long have it divided by ``factor``, with a linear ramp over the pair index between
+the pair that makes ``fast`` turns over the original context and the one that makes ``slow``;
+cos and sin are both multiplied by 0.1 ln(factor) + 1.
 """
 from __future__ import annotations
 
@@ -20,8 +26,31 @@ import torch
 from .base import Position, Rotation, Runtime, register_position
 
 
+def yarn_ramp(rotary_dim: int, theta: float, original: float, fast: float, slow: float) -> torch.Tensor:
+    """Per pair i: 0 where the frequency stays, 1 where it is divided by the factor."""
+
+    def pair_of(turns: float) -> float:
+        # the (fractional) pair index whose angle makes `turns` full turns over `original` positions
+        return rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+
+    lo = max(math.floor(pair_of(fast)), 0)
+    hi = min(math.ceil(pair_of(slow)), rotary_dim - 1)
+    i = torch.arange(rotary_dim // 2, dtype=torch.float32)
+    return torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+
+
+def table_magnitude(scaling) -> float:
+    """What cos and sin are both multiplied with."""
+    if scaling is not None and scaling.get("kind") == "yarn":
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
+
+
 def inverse_frequencies(rotary_dim: int, theta: float, scaling) -> torch.Tensor:
     inv = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    if scaling is not None and scaling.get("kind") == "yarn":
+        ramp = yarn_ramp(rotary_dim, theta, float(scaling["original"]), float(scaling["fast"]), float(scaling["slow"]))
+        return inv / float(scaling["factor"]) * ramp + inv * (1.0 - ramp)
     if scaling is not None:
         if scaling.get("kind") != "llama3":
             raise ValueError(f"rotary scaling kind {scaling.get('kind')!r} is not supported")
@@ -62,10 +91,12 @@ class Rotary(Position):
             inv = inverse_frequencies(self.rotary_dim, self.theta, self.scaling)
             pos = torch.arange(rt.max_positions, dtype=torch.float32)
             angle = torch.outer(pos, inv)  # float32 product, as the reference's table
-            _TABLES.clear()  # keep the latest only: an engine holds its own references
+            mag = table_magnitude(self.scaling)
+            while len(_TABLES) >= 4:  # keep the latest few only: an engine holds its own references
+                _TABLES.pop(next(iter(_TABLES)))
             _TABLES[key] = (
-                torch.cos(angle).contiguous().to(rt.device),
-                torch.sin(angle).contiguous().to(rt.device),
+                (torch.cos(angle) * mag).contiguous().to(rt.device),
+                (torch.sin(angle) * mag).contiguous().to(rt.device),
             )
         self.cos, self.sin = _TABLES[key]
 

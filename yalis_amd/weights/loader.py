@@ -38,7 +38,8 @@ class TensorSpec:
 
     kind: "float" or "int".
     init: how the random-weights mode fills it: ("normal", std) or
-        ("one_plus_normal", std) or ("zeros",) or ("randint", high).
+        ("one_plus_normal", std) or ("zeros",) or ("randint", high) or ("distinct", high: the
+        last axis holds different integers below high).
     """
 
     shape: Tuple[int, ...]

@@ -30,6 +30,11 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype, de
     on a GPU the same distribution from the device's generator."""
     g = torch.Generator(device=device).manual_seed(_tensor_seed(seed, name))
     kind = spec.init[0]
+    if spec.kind == "int" and kind == "distinct":
+        # every row: the last axis' many different numbers below init[1], in random order
+        lead, count = spec.shape[:-1], spec.shape[-1]
+        draws = torch.rand((*lead, spec.init[1]), generator=g, device=device, dtype=torch.float32)
+        return draws.argsort(dim=-1)[..., :count].to(torch.int32).contiguous()
     if spec.kind == "int":
         high = spec.init[1] if kind == "randint" else 2
         return torch.randint(0, high, spec.shape, generator=g, device=device, dtype=torch.int32)
