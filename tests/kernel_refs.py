@@ -230,3 +230,204 @@ def untile_cache(k_tiled, v_tiled):
     k = k_tiled.reshape(n, g, page * d)[:, :, k_at]
     v = v_tiled.reshape(n, g, page * d)[:, :, v_at]
     return k.reshape(n, g, page, d), v.reshape(n, g, d, page)
+
+
+# ------------------------------------------------------------- parts beyond the plain decoder
+# Counterparts of the kernels for branch norms, prepared / masked / finished attention heads,
+# the short convolution with its gated linear recurrence, and the mixture of experts.
+def round_rows(x, out_dtype):
+    return x if out_dtype == torch.float32 else x.to(out_dtype)
+
+
+def norm_add(residual, branch, weight, eps, unit_offset, out_dtype, expert_rows=None, expert_weight=1.0):
+    n, width = residual.shape
+    v = torch.zeros((n, width), dtype=torch.float32, device=residual.device)
+    if branch is not None:
+        v = v + branch.to(torch.float32)
+    if expert_rows is not None:
+        v = v + expert_weight * expert_rows.view(n, -1, width).sum(1)
+    residual += _rmsnorm(v, weight, eps, unit_offset)
+    return round_rows(residual, out_dtype)
+
+
+def gated_kind(activation):
+    name, consts = (activation, ()) if isinstance(activation, str) else (activation[0], tuple(activation[1:]))
+    if name not in ("silu", "gelu_tanh", "clamped_swish"):
+        raise ValueError(f"unknown activation {name!r}")
+    return name, consts
+
+
+def gated_pair(g, u, activation):
+    name, consts = gated_kind(activation)
+    if name == "silu":
+        return g * torch.sigmoid(g) * u
+    if name == "gelu_tanh":
+        return 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g**3))) * u
+    limit, slope = consts
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return g * torch.sigmoid(slope * g) * (u + 1.0)
+
+
+def gated_act_general(gu, activation, out_dtype=None, group=0):
+    inter = gu.shape[1] // 2
+    if group:
+        pairs = gu.reshape(gu.shape[0], inter // group, 2, group)
+        g = pairs[:, :, 0, :].reshape(gu.shape[0], inter).to(torch.float32)
+        u = pairs[:, :, 1, :].reshape(gu.shape[0], inter).to(torch.float32)
+    else:
+        g, u = gu[:, :inter].to(torch.float32), gu[:, inter:].to(torch.float32)
+    return gated_pair(g, u, activation).to(out_dtype or gu.dtype)
+
+
+def _turn(x, cos, sin, rot, interleaved, sign=1.0):
+    """x [..., d] float32; cos/sin [..., rot/2] broadcastable; the first rot elements turn."""
+    x = x.clone()
+    if interleaved:
+        a, b = x[..., 0:rot:2].clone(), x[..., 1:rot:2].clone()
+        x[..., 0:rot:2] = a * cos - b * sign * sin
+        x[..., 1:rot:2] = b * cos + a * sign * sin
+    else:
+        a, b = x[..., : rot // 2].clone(), x[..., rot // 2: rot].clone()
+        x[..., : rot // 2] = a * cos - b * sign * sin
+        x[..., rot // 2: rot] = b * cos + a * sign * sin
+    return x
+
+
+def qkv_prepare(qkv, n_heads, n_kv, head_dim, value_dim, positions, act_dtype, q_norm=None, k_norm=None, qk_eps=0.0,
+                rotation=None, value_norm_eps=None, value_rotation=None, k_cache=None, v_cache=None, slots=None, page_size=0):
+    n = qkv.shape[0]
+    x = qkv.to(torch.float32)
+    hd = n_heads * head_dim
+    q = x[:, :hd].reshape(n, n_heads, head_dim)
+    k = x[:, hd: hd + n_kv * head_dim].reshape(n, n_kv, head_dim)
+    v = x[:, hd + n_kv * head_dim: hd + n_kv * (head_dim + value_dim)].reshape(n, n_kv, value_dim)
+    pos = positions.long()
+    if q_norm is not None:
+        q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + qk_eps) * q_norm.to(torch.float32)
+        k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + qk_eps) * k_norm.to(torch.float32)
+    if rotation is not None:
+        c, s = rotation.cos[pos][:, None, :], rotation.sin[pos][:, None, :]
+        q = _turn(q, c, s, rotation.rotary_dim, rotation.interleaved)
+        k = _turn(k, c, s, rotation.rotary_dim, rotation.interleaved)
+    if n_kv:
+        if value_norm_eps is not None:
+            v = v * torch.rsqrt((v * v).mean(-1, keepdim=True) + value_norm_eps)
+        if value_rotation is not None:
+            v = _turn(v, value_rotation.cos[pos][:, None, :], value_rotation.sin[pos][:, None, :], value_dim, value_rotation.interleaved)
+        page, off = (slots // page_size).long(), (slots % page_size).long()
+        k_cache[page, :, off, :] = k.to(k_cache.dtype)
+        v_cache[page, :, :, off] = v.to(v_cache.dtype)
+    return q.reshape(n, hd).to(act_dtype)
+
+
+def attention_masked(q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, page_size, scale, ctx, group, window=0,
+                     keep_first=0, softcap=0.0, value_rotation=None, gate=None, gate_col=0):
+    n = q.shape[0]
+    positions, token_seq = ctx.arrays["positions"], ctx.arrays["token_seq"]
+    bt = ctx.arrays[f"block_table_g{group}"]
+    qh = q.view(n, n_heads, head_dim).to(torch.float32)
+    qpk = n_heads // n_kv
+    out = torch.empty((n, n_heads, value_dim), dtype=torch.float32, device=q.device)
+    for t in range(n):
+        pos = int(positions[t])
+        j = torch.arange(pos + 1, device=q.device)
+        if window:
+            j = j[(pos - j < window) | (j < keep_first)]
+        pages = bt[int(token_seq[t])][(j // page_size).long()].long()
+        offs = (j % page_size).long()
+        k = k_cache[pages, :, offs, :].to(torch.float32)
+        v = v_cache[pages, :, :, offs].to(torch.float32)
+        for h in range(n_heads):
+            g = h // qpk
+            s = (k[:, g, :] @ qh[t, h]) * scale
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
+            out[t, h] = torch.softmax(s, dim=0) @ v[:, g, :]
+    out = attention_finish(out, positions, n_heads, value_dim, value_rotation, gate, gate_col)
+    return out.reshape(n, n_heads * value_dim).to(q.dtype)
+
+
+def attention_finish(out, positions, n_heads, value_dim, value_rotation=None, gate=None, gate_col=0):
+    shape = out.shape
+    o = out.reshape(out.shape[0], n_heads, value_dim).to(torch.float32)
+    if value_rotation is not None:
+        pos = positions.long()
+        o = _turn(o, value_rotation.cos[pos][:, None, :], value_rotation.sin[pos][:, None, :], value_dim, value_rotation.interleaved, -1.0)
+    if gate is not None:
+        o = o * torch.sigmoid(gate[:, gate_col: gate_col + n_heads].to(torch.float32))[:, :, None]
+    return o.reshape(shape).to(out.dtype)
+
+
+def causal_conv(x, weight, bias, state, ctx):
+    n, channels = x.shape
+    taps = weight.shape[1]
+    a = ctx.arrays
+    out = torch.empty((n, channels), dtype=torch.float32, device=x.device)
+    for t in range(n):
+        seq = int(a["token_seq"][t])
+        local = t - int(a["seq_qstart"][seq])
+        acc = bias.to(torch.float32).clone() if bias is not None else torch.zeros(channels)
+        for j in range(taps):
+            back = taps - 1 - j
+            if local - back >= 0:
+                v = x[t - back].to(torch.float32)
+            else:
+                v = state[int(a["state_slots"][seq]), taps - 1 + local - back].to(torch.float32)
+            acc = acc + weight[:, j].to(torch.float32) * v
+        out[t] = acc
+    return out.to(x.dtype)
+
+
+def rglru(u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx):
+    n, channels = u.shape
+    blocks = wa_t.shape[0]
+    a = ctx.arrays
+    uf = u.to(torch.float32).view(n, blocks, -1)
+    r = torch.sigmoid(torch.einsum("tbi,bio->tbo", uf, wa_t.to(torch.float32)).reshape(n, channels) + ba.to(torch.float32))
+    i = torch.sigmoid(torch.einsum("tbi,bio->tbo", uf, wi_t.to(torch.float32)).reshape(n, channels) + bi.to(torch.float32))
+    log_a = -rate * r * torch.nn.functional.softplus(lam.to(torch.float32))
+    av = torch.exp(log_a)
+    bv = torch.sqrt(-torch.expm1(2.0 * log_a)) * i * u.to(torch.float32)
+    yf = y.to(torch.float32)
+    gelu = 0.5 * yf * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (yf + 0.044715 * yf**3)))
+    out = torch.empty((n, channels), dtype=torch.float32, device=u.device)
+    for s in range(a["seq_qstart"].numel()):
+        q0, ql, slot = int(a["seq_qstart"][s]), int(a["seq_qlen"][s]), int(a["state_slots"][s])
+        S = s_state[slot].clone()
+        for t in range(q0, q0 + ql):
+            S = av[t] * S + bv[t]
+            out[t] = S * gelu[t]
+        s_state[slot] = S
+        if taps > 1:
+            hist = torch.cat([conv_state[slot], x[q0: q0 + ql].to(conv_state.dtype)], dim=0)
+            conv_state[slot] = hist[-(taps - 1):]
+    return out.to(u.dtype)
+
+
+def moe_experts(x, token_ids, table, w_gate_up, w_down, activation):
+    n, hidden = x.shape
+    top = table.shape[1]
+    rows = torch.empty((n * top, hidden), dtype=torch.float32, device=x.device)
+    xf = x.to(torch.float32)
+    for t in range(n):
+        for k in range(top):
+            e = int(table[int(token_ids[t]), k])
+            g = w_gate_up[e, 0].to(torch.float32) @ xf[t]
+            u = w_gate_up[e, 1].to(torch.float32) @ xf[t]
+            yv = gated_pair(g, u, activation).to(x.dtype).to(torch.float32)
+            rows[t * top + k] = w_down[e].to(torch.float32) @ yv
+    return rows
+
+
+RefOps.round_rows = staticmethod(round_rows)
+RefOps.norm_add = staticmethod(norm_add)
+RefOps.gated_kind = staticmethod(gated_kind)
+RefOps.gated_act = staticmethod(gated_act_general)
+RefOps.gate_up_act = staticmethod(lambda x, w, group, activation, out_dtype: gated_act_general(linear(x, w, out_dtype), activation, out_dtype, group))
+RefOps.qkv_prepare = staticmethod(qkv_prepare)
+RefOps.attention_masked = staticmethod(attention_masked)
+RefOps.attention_finish = staticmethod(attention_finish)
+RefOps.causal_conv = staticmethod(causal_conv)
+RefOps.rglru = staticmethod(rglru)
+RefOps.moe_experts = staticmethod(moe_experts)

@@ -81,7 +81,8 @@ def attention_mixer(h, m, w, pre, eps):
     fv = rot["base"] ** (-2.0 * torch.arange(dv // 2, dtype=F) / dv)
     vang = pos[:, None] * fv[None, :]
     v = rotate_halves(v, vang)
-    mask = visible(T, m["mask"]["size"], m["mask"]["keep_first"])
+    mask = m.get("mask") or {}
+    mask = visible(T, mask.get("size") or T, mask.get("keep_first", 0))
     out = torch.empty(H, T, dv, dtype=F)
     for hh in range(H):
         g = hh // (H // G)
