@@ -159,7 +159,7 @@ def make_engine(cfg: dict, max_batch: int, ctx_cap: int, graphs: bool = True, pa
     from yalis_amd.config.runtime import EngineConfig
 
     pages_per_req = -(-ctx_cap // page)
-    max_len = min(cfg["max_position_embeddings"], pages_per_req * page)
+    max_len = min(cfg.get("max_position_embeddings", 1 << 30), pages_per_req * page)
     engine = EngineConfig(
         page_size=page, num_pages=-(-pool_tokens // page) if pool_tokens else pages_per_req * max_batch, max_num_seqs=max_batch,
         max_model_len=max_len, max_num_batched_tokens=8192, dtype="bfloat16", decode_graphs=graphs,
@@ -377,8 +377,175 @@ def breakdown(runner, shape: Shape, gen, batch: int, prompt_len: int, prefill_le
     return out
 
 
+# ------------------------------------------------------- another design beside its closest model
+def _op_costs(ops, hb):
+    """name -> function(args, kwargs, result) -> (flops, bytes): what a call into the kernel library has
+    to compute and to move at the least.  ``hb`` is a function giving the step's host batch."""
+    def nbytes(*ts):
+        return sum(t.numel() * t.element_size() for t in ts if hasattr(t, "numel"))
+
+    def visible(window, keep):
+        b = hb()
+        total = 0
+        for ctx, ql in zip(b.seq_ctx.tolist(), b.seq_qlen.tolist()):
+            for p in range(ctx - ql, ctx):
+                total += p + 1 if not window else min(p + 1, window + min(keep, max(0, p + 1 - window)))
+        return total
+
+    def linear(a, kw, out):
+        x, w = a[0], a[1]
+        m, k, n = x.shape[0], w.shape[1], w.shape[0]
+        return 2.0 * m * n * k, 2.0 * (m * k + n * k + m * n)
+
+    def moe(a, kw, out):
+        x, table, wgu, wd = a[0], a[2], a[3], a[4]
+        m, top, experts = x.shape[0], table.shape[1], wgu.shape[0]
+        per_expert = wgu[0].numel() + wd[0].numel()
+        return 2.0 * m * top * per_expert, 2.0 * min(m * top, experts) * per_expert + nbytes(x) * (1 + top) + 4.0 * m * top * x.shape[1]
+
+    def attention_masked(a, kw, out):
+        q, heads, kv, d, dv = a[0], a[1], a[2], a[3], a[4]
+        keys = visible(kw.get("window", 0), kw.get("keep_first", 0))
+        b = hb()
+        cached = sum(min(c, (kw.get("window") or c) + kw.get("keep_first", 0)) for c in b.seq_ctx.tolist())
+        return 2.0 * heads * (d + dv) * keys, 2.0 * kv * (d + dv) * cached + nbytes(q) * 2
+
+    def attention(a, kw, out):
+        qkv, heads, kv, d = a[0], a[1], a[2], a[3]
+        keys = visible(a[8], 0)
+        b = hb()
+        return 4.0 * heads * d * keys, 4.0 * kv * d * sum(b.seq_ctx.tolist()) + 4.0 * qkv.shape[0] * heads * d
+
+    def rglru(a, kw, out):
+        u, wa = a[0], a[3]
+        return 4.0 * u.shape[0] * u.shape[1] * wa.shape[1], nbytes(u) * 4 + nbytes(wa) * 2
+
+    def moved(a, kw, out):
+        return 0.0, float(nbytes(*a, *kw.values()) + (nbytes(out) if hasattr(out, "numel") else 0))
+
+    return {"linear": linear, "gate_up_act": linear, "moe_experts": moe, "attention_masked": attention_masked, "attention": attention,
+            "rglru": rglru, "norm_add": moved, "add_rmsnorm": moved, "gather_add_rmsnorm": moved, "qkv_prepare": moved,
+            "rope_append": moved, "causal_conv": moved, "gated_act": moved, "round_rows": moved, "embed": moved}
+
+
+def per_op_times(runner, vocab: int, gen, batch: int, prompt_len: int, prefill_len: int):
+    """Time and bound of every kind of call into the kernel library, for a prefill of ``prefill_len``
+    tokens and for a decode step of ``batch`` requests behind ``prompt_len``-token prompts: {phase:
+    {op: [microseconds, bound in microseconds, time / bound]}}; the bound is max(bytes / 8 TB/s,
+    flops / 2.5 PFLOP/s) of what the call must move and compute at the least."""
+    import torch
+
+    from yalis_amd.engine.step import StepEntry
+
+    ops = runner.rt.ops
+    costs = _op_costs(ops, lambda: runner.last_host_batch)
+    spans, depth = [], [0]
+    current = {}
+
+    def timed(name, fn):
+        def call(*a, **kw):
+            if depth[0]:
+                return fn(*a, **kw)
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            depth[0] += 1
+            start.record()
+            try:
+                out = fn(*a, **kw)
+            finally:
+                stop.record()
+                depth[0] -= 1
+            spans.append((name, start, stop, costs[name](a, kw, out)))
+            return out
+        return call
+
+    saved = {name: getattr(ops, name) for name in costs if hasattr(ops, name)}
+    for name, fn in saved.items():
+        setattr(ops, name, timed(name, fn))
+    graphs, runner.use_graphs = runner.use_graphs, False
+    # the host batch of the running step, for the attention's counts: set before the model runs
+    real_forward = runner.model.forward
+
+    def forward(ctx):
+        runner.last_host_batch = ctx.host
+        return real_forward(ctx)
+
+    runner.model.forward = forward
+    out = {}
+
+    def collect(n):
+        sums = {}
+        for name, a, b, (flops, nbytes) in spans:
+            t, bound = sums.setdefault(name, [0.0, 0.0])
+            sums[name] = [t + a.elapsed_time(b) * 1e3 / n, bound + 1e6 * max(nbytes / (HBM_GBPS * 1e9), flops / BF16_FLOPS) / n]
+        return {k: [round(t, 1), round(bd, 1), round(t / bd, 1) if bd else None] for k, (t, bd) in sorted(sums.items())}
+
+    try:
+        prompt = torch.randint(0, vocab, (prefill_len,), generator=gen).tolist()
+        for i in range(3):
+            spans.clear()
+            assert runner.admit(3000 + i) and runner.reserve(3000 + i, prefill_len)
+            ops.argmax(runner.step([StepEntry(3000 + i, prompt, [prefill_len - 1])])).tolist()
+            torch.cuda.synchronize()
+            runner.release(3000 + i)
+        out["prefill_us"] = collect(1)
+        toks = []
+        for r in range(batch):
+            assert runner.admit(r)
+            p = torch.randint(0, vocab, (prompt_len,), generator=gen).tolist()
+            assert runner.reserve(r, len(p) + 8)
+            toks.append(ops.argmax(runner.step([StepEntry(r, p, [len(p) - 1])])).tolist()[0])
+        for i in range(5):
+            if i == 1:
+                spans.clear()
+            toks = ops.argmax(runner.step([StepEntry(r, [toks[r]], [0]) for r in range(batch)])).tolist()
+            torch.cuda.synchronize()
+        out["decode_us"] = collect(4)
+        for r in range(batch):
+            runner.release(r)
+    finally:
+        runner.use_graphs = graphs
+        runner.model.forward = real_forward
+        for name, fn in saved.items():
+            setattr(ops, name, fn)
+    return out
+
+
+def design_compare(args) -> int:
+    """Prefill and decode throughput of another design at a few layer sizes (random weights), beside
+    the Llama configuration of equal size; one JSON line a size."""
+    import torch
+
+    from yalis_amd.models.presets import llama_like
+
+    sizes = {"suranex": ("suranex-2k", "suranex-4k")}[args.design]
+    for name in sizes:
+        label, cfg = SHAPES[name]
+        line = {"design": args.design, "shape": label, "batch": args.batch, "prompt_len": args.prompt_len, "prefill_len": args.prefill_len,
+                "dtype": "bf16", "data": "synthetic: random bf16 weights, seeded uniform-random token ids"}
+        for who, c in (("design", cfg), ("llama_of_equal_size", llama_like(cfg))):
+            gen = torch.Generator().manual_seed(0)
+            vocab = c.get("vocab", c.get("vocab_size"))
+            steps = args.steps
+            ctx_cap = max(args.prompt_len + steps + args.warmup + 16, args.prefill_len)
+            engine = make_engine(dict(c), max(args.batch, 1), ctx_cap)
+            runner = engine.runner
+            pf, _ = prefill_run(runner, vocab, gen, args.prefill_len, runs=4)
+            dt, _ = decode_run(runner, vocab, gen, args.batch, args.prompt_len, steps, args.warmup)
+            entry = {"layers": len(c["layers"]) if "layers" in c else c["num_hidden_layers"],
+                     "prefill_tok_s": round(args.prefill_len / pf, 1), "prefill_ms": round(1e3 * pf, 3),
+                     "decode_tok_s": round(args.batch * steps / dt, 1), "decode_ms_per_step": round(1e3 * dt / steps, 4)}
+            entry["ops"] = per_op_times(runner, vocab, gen, args.batch, args.prompt_len, args.prefill_len)
+            line[who] = entry
+            del runner, engine
+            torch.cuda.empty_cache()
+        print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", choices=("suranex",), default=None,
+                    help="measure instead another design's prefill and decode at a few layer sizes, beside the Llama configuration of equal size, with the time and the bound of every kind of kernel")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=32)
     ap.add_argument("--warmup", type=int, default=4)
@@ -402,6 +569,8 @@ def main() -> int:
 
     import torch
 
+    if args.design:
+        return design_compare(args)
     if args.probe:
         return machine_probe(SHAPES[args.shape][1])
     if args.sample:

@@ -45,6 +45,37 @@ TINY_B = {
     "max_position_embeddings": 256, "tie_word_embeddings": True,
 }
 
+
+
+def suranex_shape(width: int, vocab: int, heads: int, kv_heads: int, dim: int, window: int, recurrent_width: int, blocks: int,
+                  experts: int, top: int, ff: int, shared_ff: int, pattern=("attention", "attention", "rglru"), repeats: int = 2) -> dict:
+    """A Suranex config.json of the given layer sizes: ``pattern`` repeated ``repeats`` times, every
+    layer with a mixture of experts and a shared expert."""
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 50.0,
+           "mask": {"size": window, "keep_first": 4},
+           "rot": {"base": 10000.0, "dims": dim, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    rec = {"width": recurrent_width, "blocks": blocks, "conv": 4}
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff, "limit": 7.0},
+           "shared": {"ff": shared_ff, "limit": 7.0}}
+    layers = [{"type": kind, "mixer": dict(att if kind == "attention" else rec), "mlp": dict(mlp)} for kind in pattern * repeats]
+    return {"architecture": "Suranex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": layers}
+
+
+def llama_like(suranex: dict) -> dict:
+    """The Llama configuration of equal size: the same width, layer count, vocabulary and (first
+    attention layer's) heads, a feed-forward as wide as what a token uses of the mixture (its top
+    experts and the shared one)."""
+    att = next(layer["mixer"] for layer in suranex["layers"] if layer["type"] == "attention")
+    mlp = next(layer["mlp"] for layer in suranex["layers"] if layer["mlp"] is not None)
+    inter = mlp["router"]["top"] * mlp["expert"]["ff"] + (mlp["shared"]["ff"] if mlp.get("shared") else 0)
+    return dict(LLAMA3_8B, hidden_size=suranex["width"], num_hidden_layers=len(suranex["layers"]), num_attention_heads=att["heads"],
+                num_key_value_heads=att["kv_heads"], head_dim=att["dim"], intermediate_size=inter, vocab_size=suranex["vocab"])
+
+
+SURANEX_2K = suranex_shape(2048, 32768, 16, 4, 128, 1024, 2560, 10, 16, 2, 1024, 2048)
+SURANEX_4K = suranex_shape(4096, 65536, 32, 8, 128, 2048, 5120, 20, 32, 4, 1024, 4096, repeats=1)
+SURANEX_TINY = suranex_shape(64, 256, 4, 2, 16, 24, 96, 3, 4, 2, 32, 48, repeats=1)
+
 # name -> (what to call it, config.json dictionary)
 SHAPES: Dict[str, Tuple[str, dict]] = {
     "8b": ("Llama-3-8B", LLAMA3_8B),
@@ -53,6 +84,9 @@ SHAPES: Dict[str, Tuple[str, dict]] = {
     "70b": ("Llama-3.1-70B", LLAMA31_70B),
     "tiny-a": ("tiny Llama A", TINY_A),
     "tiny-b": ("tiny Llama B", TINY_B),
+    "suranex-2k": ("Suranex, width 2,048", SURANEX_2K),
+    "suranex-4k": ("Suranex, width 4,096", SURANEX_4K),
+    "suranex-tiny": ("tiny Suranex", SURANEX_TINY),
 }
 
 
