@@ -128,6 +128,26 @@ extern "C" int yk_attn_generic(const void* q, int q_stride, void* out, const voi
 }
 
 // ------------------------------------------------------------------------ matrix cores
+// Options of the matrix-core kernels beyond the plain causal window (their EXT instantiations; the
+// plain ones are compiled without): the first `keep_first` keys of a request stay visible below
+// the window, and a score s (times the scale) is squashed to cap * tanh(s / cap).
+//
+// Kept first keys add blocks of 64 keys in front of the window's: a kernel numbers the blocks it
+// walks "virtually", the window's blocks by their own number and the n_first blocks of kept keys
+// just below the window's first block; ext_block gives the block a virtual number stands for.
+__device__ __forceinline__ int ext_first_blocks(int keep_first, int window, int lo) {
+  return window > 0 && keep_first > 0 ? min((keep_first + 63) / 64, lo / 64) : 0;
+}
+__device__ __forceinline__ int ext_block(int vb, int first_window_block, int n_first) {
+  return vb >= first_window_block ? vb : vb - (first_window_block - n_first);
+}
+// s * scale squashed, returned in the raw score's units (the kernels multiply by the scale later):
+// (cap / scale) * tanh(s * scale / cap), the tanh from one exp2 and one division
+__device__ __forceinline__ float ext_squash(float s, float cap_over_scale, float scale_over_cap_2log2e) {
+  const float e = __builtin_amdgcn_exp2f(s * scale_over_cap_2log2e);  // e^(2x); inf and 0 at the ends give +-1
+  return cap_over_scale * (1.f - __fdividef(2.f, 1.f + e));
+}
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -222,13 +242,15 @@ __device__ __forceinline__ float rope_src_add8(float acc, const float (&d)[8], i
   return acc;
 }
 
-template <int D, int W, bool TILED, int SRC>
+template <int D, int W, bool TILED, int SRC, bool EXT = false>
 __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* k_cache, const bf16_t* v_cache,  // (written too, with ROPE: the token's own slot)
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
-    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, RopeSrc rs) {
+    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, RopeSrc rs, int keep_first_arg = 0,
+    float cap_over_scale = 0.f, float scale_over_cap_2log2e = 0.f) {
+  const int keep_first = EXT ? keep_first_arg : 0;
   constexpr int KS = D / 32;  // matrix-core steps over the head dimension
   constexpr int DT = D / 16;  // output tiles over the head dimension
   constexpr bool ROPE = SRC != 0;  // SRC 0: queries from `q`; 1, 2: rotary + append in here (rope_src_load8)
@@ -248,7 +270,11 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   const int lo_c = window > 0 ? max(0, pos_c - window + 1) : 0;
   const int hi = pos0 + ntok;
   const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
-  const int kb_lo = lo / 64, kb_hi = (hi + 63) / 64;
+  // (blocks are numbered virtually: those of kept first keys sit just below the window's first)
+  const int win_lo = lo / 64;
+  const int n_first = EXT ? ext_first_blocks(keep_first, window, lo) : 0;
+#define ATT_BLK(VB) (EXT ? ext_block((VB), win_lo, n_first) : (VB))
+  const int kb_lo = win_lo - n_first, kb_hi = (hi + 63) / 64;
   const int per_split = (kb_hi - kb_lo + n_splits - 1) / n_splits;
   const int wg_lo = kb_lo + blockIdx.z * per_split;
   const int wg_hi = min(kb_hi, wg_lo + per_split);
@@ -278,12 +304,12 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   auto page_of = [&](int key) { return max(0, bt[min(key / page_size, last_page_col)]); };
 
   AFrag8 kf[2][2][KS];
-#define ATT_LOAD_K(KB) ATT_LOAD_K_AT(KB, page_of((KB) * 64))
+#define ATT_LOAD_K(KB) ATT_LOAD_K_AT(KB, page_of(ATT_BLK(KB) * 64))
   // PAGE0: the page of the block's first key, for tiled pages (looked up by the caller)
 #define ATT_LOAD_K_AT(KB, PAGE0)                                                                  \
   {                                                                                                \
   if (TILED) {                                                                                     \
-    const int key0 = (KB) * 64;                                                                    \
+    const int key0 = ATT_BLK(KB) * 64;                                                             \
     const bf16_t* kp = k_cache + (static_cast<size_t>(PAGE0) * n_kv + g) * page_size * D +         \
                        static_cast<size_t>(key0 % page_size) * D + 8 * lane;                       \
     _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
@@ -300,7 +326,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
       if (mine((KB), u)) {                                                                         \
         _Pragma("unroll") for (int sb = 0; sb < 2; ++sb) {                                         \
-          const int key = (KB) * 64 + 32 * u + krow + 4 * sb;                                     \
+          const int key = ATT_BLK(KB) * 64 + 32 * u + krow + 4 * sb;                              \
           const bf16_t* kp = k_cache + ((static_cast<size_t>(page_of(key)) * n_kv + g) * page_size + key % page_size) * D + 8 * gq; \
           _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                       \
               kf[u][sb][ks].u = *reinterpret_cast<const u32x4_t*>(kp + 32 * ks);                  \
@@ -318,7 +344,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 #define ATT_LOAD_V_AT(KB, PAGE0)                                                                   \
   {                                                                                                \
   if (TILED) {                                                                                     \
-    const int key0 = (KB) * 64;                                                                    \
+    const int key0 = ATT_BLK(KB) * 64;                                                             \
     const bf16_t* vp = v_cache + (static_cast<size_t>(PAGE0) * n_kv + g) * D * page_size +         \
                        static_cast<size_t>(key0 % page_size) * D + 8 * lane;                       \
     _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
@@ -332,7 +358,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   } else {                                                                                         \
     _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
       if (mine((KB), u)) {                                                                         \
-        const int key = (KB) * 64 + 32 * u + 8 * gq;                                               \
+        const int key = ATT_BLK(KB) * 64 + 32 * u + 8 * gq;                                        \
         const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key)) * n_kv + g) * D * page_size + key % page_size; \
         _Pragma("unroll") for (int dt = 0; dt < DT; ++dt)                                          \
             vf[u][dt].u = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(16 * dt + r) * page_size); \
@@ -379,7 +405,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     const size_t src_split_stride = rs.split_stride;
     // the page of the first block is asked for first: the keys' addresses wait for it, and a
     // wait for an older load leaves the younger ones in flight
-    const int first_page = my_lo < my_hi ? page_of(my_lo * 64) : 0;
+    const int first_page = my_lo < my_hi ? page_of(ATT_BLK(my_lo) * 64) : 0;
     // one round; LOAD_K: the first block's keys are asked for while the round's rows are on
     // their way (the first round is straight-line code: its loads are all issued before the
     // first of them is waited for; rows of more than eight slices finish in a loop)
@@ -479,7 +505,8 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   }
   for (int kb = my_lo; kb < my_hi; ++kb) {
     const bool mine0 = mine(kb, 0), mine1 = mine(kb, 1);
-    if (!(ROPE && kb == my_lo)) ATT_LOAD_V_AT(kb, page_of(kb * 64))  // (ROPE: the first block's are on their way)
+    const int akb = ATT_BLK(kb);  // the block of keys that the virtual number stands for
+    if (!(ROPE && kb == my_lo)) ATT_LOAD_V_AT(kb, page_of(akb * 64))  // (ROPE: the first block's are on their way)
     // scores
     f32x4_t s[2][2];
 #pragma unroll
@@ -498,7 +525,16 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     float tmax = -INFINITY;
     // a block that every column sees whole needs no mask (columns that stand for nothing
     // compute on zeros and are never stored)
-    const bool whole = mine0 && mine1 && kb * 64 + 63 <= pos0 && (window == 0 || kb * 64 >= max(0, pos0 + ntok - window));
+    const bool whole = mine0 && mine1 && akb * 64 + 63 <= pos0 &&
+                       (window == 0 || akb * 64 >= max(0, pos0 + ntok - window) || (EXT && akb * 64 + 64 <= keep_first));
+    if (EXT && cap_over_scale > 0.f) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s[u][sb][i] = ext_squash(s[u][sb][i], cap_over_scale, scale_over_cap_2log2e);
+    }
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -506,8 +542,11 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           if (!whole) {
-            const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
-            const bool ok = col_ok && key <= pos_c && key >= lo_c && (u == 0 ? mine0 : mine1);
+            const int key = akb * 64 + 32 * u + 8 * gq + 4 * sb + i;
+            // (a lower bound per key; written as `key >= lo_c || key < keep_first` this kernel let the key
+            // just below the window through in one of its four rows, which the test with one towering key shows)
+            const int lo_k = (EXT && key < keep_first) ? 0 : lo_c;  // kept first keys have no lower bound
+            const bool ok = col_ok && key <= pos_c && key >= lo_k && (u == 0 ? mine0 : mine1);
             if (!ok) s[u][sb][i] = -INFINITY;
           }
           tmax = fmaxf(tmax, s[u][sb][i]);
@@ -542,15 +581,15 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     }
     // values of keys that do not exist yet, or that lie below the window (their pages may have
     // been given back), may be anything: zero them (the last and the first block only)
-    if (kb * 64 + 64 > hi || kb * 64 < lo) {
+    if (akb * 64 + 64 > hi || akb * 64 < lo) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const int key = kb * 64 + 32 * u + 8 * gq;
+        const int key = akb * 64 + 32 * u + 8 * gq;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (key + e >= hi || key + e < lo) vf[u][dt].h[e] = 0;
+            if (key + e >= hi || (key + e < lo && key + e >= keep_first)) vf[u][dt].h[e] = 0;
       }
     }
     if (ROPE && makes_kv && kb == kb_new && gq == new_gq) {
@@ -575,6 +614,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
       for (int dt = 0; dt < DT; ++dt)
         acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[u][dt].v, pf[u].v, acc[dt], 0, 0, 0);
   }
+#undef ATT_BLK
 #undef ATT_LOAD_K
 #undef ATT_LOAD_K_AT
 #undef ATT_LOAD_V_AT
@@ -649,14 +689,16 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 // registers, two workgroups a CU) stage every block through LDS for twice the columns and
 // win where many tiles each meet thousands of keys (measured on the 8B shape: 2,048 tokens
 // against 8,192 cached 383 us against 499, a whole 2,048-token prompt 99 us against 80).
-template <int D, bool TILED, int CT>
+template <int D, bool TILED, int CT, bool EXT>
 __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
-    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, int pages_lds_limit) {
+    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, int pages_lds_limit, int keep_first_arg,
+    float cap_over_scale, float scale_over_cap_2log2e) {
   constexpr int KS = D / 32, DT = D / 16;
+  const int keep_first = EXT ? keep_first_arg : 0;
   constexpr int KROW = D + 8;   // bf16 elements per parked key row
   constexpr int VROW = 64 + 8;  // bf16 elements per parked value row
   constexpr int PP = D / 32;    // 16-byte pieces of keys (and of values) per thread and block
@@ -693,7 +735,11 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
   const int wave_hi = min(hi, tile_pos0 + wave_tok0 + CT * tpt);  // keys this wave may need
   // the workgroup's share of the key blocks when a launch splits them (blockIdx.y): few long
   // tiles against a long context would otherwise leave most of the GPU idle
-  const int all_lo = lo / 64, all_hi = (hi + 63) / 64;
+  // (blocks are numbered virtually: those of kept first keys sit just below the window's first)
+  const int win_lo = lo / 64;
+  const int n_first = EXT ? ext_first_blocks(keep_first, window, lo) : 0;
+  auto block_of = [&](int vb) { return EXT ? ext_block(vb, win_lo, n_first) : vb; };
+  const int all_lo = win_lo - n_first, all_hi = (hi + 63) / 64;
   const int per_split = (all_hi - all_lo + n_splits - 1) / n_splits;
   const int kb_lo = all_lo + blockIdx.y * per_split, kb_hi = min(all_hi, kb_lo + per_split);
   const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
@@ -702,7 +748,7 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
   // would put a dependent memory round trip before every load)
   constexpr int PAGES_LDS = 2048;
   __shared__ int32_t pages_s[PAGES_LDS];
-  const int first_col = min(last_page_col, max(0, kb_lo) * 64 / page_size);
+  const int first_col = min(last_page_col, max(0, block_of(kb_lo)) * 64 / page_size);
   // (pages_lds_limit: at most PAGES_LDS; tests lower it to walk the other way with short tables)
   const bool pages_in_lds = last_page_col - first_col < min(PAGES_LDS, pages_lds_limit);
   if (pages_in_lds)
@@ -765,8 +811,13 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
   const size_t page_elems = static_cast<size_t>(n_kv) * page_size * D;
   // (tiled pages: the blocks are fetched in their order, so the column of the block table and
   // the place within the page are stepped along instead of divided out for every block)
-  int pf_col = page_col(kb_lo * 64), pf_off = page_off(kb_lo * 64);
-#define PF_LOAD(KB)                                                                                \
+  int pf_col = page_col(block_of(kb_lo) * 64), pf_off = page_off(block_of(kb_lo) * 64);
+#define PF_LOAD(VB)                                                                                \
+  const int KB = block_of(VB);                                                                      \
+  if (EXT && TILED) {  /* the walk may jump from the kept first keys to the window */               \
+    pf_col = page_col(KB * 64);                                                                     \
+    pf_off = page_off(KB * 64);                                                                     \
+  }                                                                                                 \
   if (TILED) {                                                                                      \
     const int page = pages_in_lds ? pages_s[pf_col - first_col] : max(0, bt[pf_col]);               \
     const size_t base = static_cast<size_t>(page) * page_elems + static_cast<size_t>(g) * page_size * D + \
@@ -796,7 +847,8 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
   }
 
   if (kb_lo < kb_hi) { PF_LOAD(kb_lo) }
-  for (int kb = kb_lo; kb < kb_hi; ++kb) {
+  for (int vb = kb_lo; vb < kb_hi; ++vb) {
+    const int kb = block_of(vb);
     __syncthreads();  // every wave is done with the previous block
 #pragma unroll
     for (int p = 0; p < PP; ++p) {
@@ -814,14 +866,14 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
           f.u = v;
 #pragma unroll
           for (int i = 0; i < 8; ++i)
-            if (key + i >= hi || key + i < lo) f.h[i] = 0;
+            if (key + i >= hi || (key + i < lo && key + i >= keep_first)) f.h[i] = 0;
           v = f.u;
         }
         *reinterpret_cast<u32x4_t*>(&vs[v_dim[p]][v_key[p]]) = v;
       }
     }
     __syncthreads();
-    if (kb + 1 < kb_hi) { PF_LOAD(kb + 1) }  // in flight while this block is worked on
+    if (vb + 1 < kb_hi) { PF_LOAD(vb + 1) }  // in flight while this block is worked on
     const int key0 = kb * 64;
     if (key0 >= wave_hi) continue;  // nothing of this block is visible to this wave
 
@@ -843,7 +895,18 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
       }
     // keys that every column sees whole need no mask (columns that stand for nothing
     // compute on zeros and are never stored)
-    const bool whole = key0 + 63 <= (tile_pos0 + wave_tok0) && (window == 0 || key0 >= max(0, wave_hi - window));
+    const bool whole = key0 + 63 <= (tile_pos0 + wave_tok0) &&
+                       (window == 0 || key0 >= max(0, wave_hi - window) || (EXT && key0 + 64 <= keep_first));
+    if (EXT && cap_over_scale > 0.f) {
+#pragma unroll
+      for (int c = 0; c < CT; ++c)
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[c][u][sb][i] = ext_squash(s[c][u][sb][i], cap_over_scale, scale_over_cap_2log2e);
+    }
     AFrag8 pf[CT][2];
     float alpha[CT];
     bool grew = false;  // some column's maximum rose: only then the running sums need rescaling
@@ -859,7 +922,8 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int key = key0 + 32 * u + 8 * gq + 4 * sb + i;
-              const bool ok = col_ok[c] && key <= pos_c[c] && key >= lo_c[c];
+              const int lo_k = (EXT && key < keep_first) ? 0 : lo_c[c];  // kept first keys have no lower bound
+              const bool ok = col_ok[c] && key <= pos_c[c] && key >= lo_k;
               s[c][u][sb][i] = ok ? s[c][u][sb][i] : -INFINITY;
             }
       }
@@ -1004,7 +1068,7 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
                                     const int32_t* block_table, int table_width, int page_size,
                                     int head_dim, int n_heads, int n_kv, float scale, int window,
                                     int n_splits, int col_tiles, float* workspace, size_t workspace_floats,
-                                    int pages_lds_limit, hipStream_t stream) {
+                                    int pages_lds_limit, int keep_first, float softcap, hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma_prefill: bad head counts");
   YK_REQUIRE(col_tiles == 1 || col_tiles == 2, "attn_mfma_prefill: a wave has 1 or 2 column tiles");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma_prefill: head_dim must be 64 or 128");
@@ -1015,7 +1079,11 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
              "attn_mfma_prefill: cache must be 16-byte aligned");
   YK_REQUIRE(window >= 0 && table_width > 0, "attn_mfma_prefill: bad window or table");
   YK_REQUIRE(scale > 0.f, "attn_mfma_prefill: the score scale must be positive");
+  YK_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attn_mfma_prefill: keep_first and softcap must not be negative");
   if (n_tiles == 0) return 0;
+  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f;
+  const float cap_over_scale = softcap > 0.f ? softcap / scale : 0.f;
+  const float scale_over_cap = softcap > 0.f ? scale / softcap * 2.f * 1.4426950408889634f : 0.f;
   const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
   const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
   YK_REQUIRE(static_cast<long long>(n_tiles) * n_kv * chunks <= 0x7fffffffLL, "attn_mfma_prefill: too many tiles for one launch");
@@ -1029,12 +1097,16 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
 #define YK_PF_ARGS                                                                                           \
   static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),     \
       static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt,     \
-      chunks, scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit
+      chunks, scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit, keep_first, cap_over_scale, scale_over_cap
 #define YK_PF(DD, BIP)                                                                                       \
-  if (col_tiles == 2)                                                                                        \
-    attn_mfma_prefill_kernel<DD, BIP, 2><<<grid, block, 0, stream>>>(YK_PF_ARGS);                            \
+  if (ext && col_tiles == 2)                                                                                 \
+    attn_mfma_prefill_kernel<DD, BIP, 2, true><<<grid, block, 0, stream>>>(YK_PF_ARGS);                      \
+  else if (ext)                                                                                              \
+    attn_mfma_prefill_kernel<DD, BIP, 1, true><<<grid, block, 0, stream>>>(YK_PF_ARGS);                      \
+  else if (col_tiles == 2)                                                                                   \
+    attn_mfma_prefill_kernel<DD, BIP, 2, false><<<grid, block, 0, stream>>>(YK_PF_ARGS);                     \
   else                                                                                                       \
-    attn_mfma_prefill_kernel<DD, BIP, 1><<<grid, block, 0, stream>>>(YK_PF_ARGS)
+    attn_mfma_prefill_kernel<DD, BIP, 1, false><<<grid, block, 0, stream>>>(YK_PF_ARGS)
   const bool bip = cache_is_tiled(YK_BF16, head_dim, page_size);
   if (head_dim == 64) {
     if (bip) { YK_PF(64, true); } else { YK_PF(64, false); }
@@ -1063,8 +1135,14 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             const int32_t* tiles, int n_tiles, const int32_t* block_table, int table_width,
                             int page_size, int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
-                            int leave_splits, const RopeSrc* rope, bool rope_f32, hipStream_t stream) {
+                            int leave_splits, const RopeSrc* rope, bool rope_f32, hipStream_t stream, int keep_first = 0,
+                            float softcap = 0.f) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
+  YK_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attn_mfma: keep_first and softcap must not be negative");
+  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f;
+  YK_REQUIRE(!(ext && rope), "attn_mfma: kept first keys and squashed scores are not offered with rotary inside the launch");
+  const float cap_over_scale = softcap > 0.f ? softcap / scale : 0.f;
+  const float scale_over_cap = softcap > 0.f ? scale / softcap * 2.f * 1.4426950408889634f : 0.f;
   YK_REQUIRE(n_waves == 1 || n_waves == 4, "attn_mfma: a workgroup has 1 or 4 waves");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma: head_dim must be 64 or 128");
   YK_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page_size must be a multiple of 16");
@@ -1099,7 +1177,16 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
     if (n_waves == 1) attn_mfma_kernel<DD, 1, false, RR><<<grid, block, 0, stream>>>(YK_ARGS);     \
     else attn_mfma_kernel<DD, 4, false, RR><<<grid, block, 0, stream>>>(YK_ARGS);                  \
   }
+#define YK_LAUNCH_EXT(DD)                                                                          \
+  if (tiled) {                                                                                     \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
+    else attn_mfma_kernel<DD, 4, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
+  } else {                                                                                         \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
+    else attn_mfma_kernel<DD, 4, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
+  }
 #define YK_LAUNCH(DD)                                                                              \
+  if (ext) { YK_LAUNCH_EXT(DD) } else                                                              \
   if (!rope) { YK_LAUNCH_R(DD, 0) } else if (rope_f32) { YK_LAUNCH_R(DD, 2) } else { YK_LAUNCH_R(DD, 1) } \
   if (yk_check_launch("attn_mfma")) return -1;                                                     \
   if (n_splits > 1 && !leave_splits) {                                                             \
@@ -1113,6 +1200,7 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
     YK_LAUNCH(128)
   }
 #undef YK_LAUNCH
+#undef YK_LAUNCH_EXT
 #undef YK_LAUNCH_R
 #undef YK_ARGS
   return 0;
@@ -1123,10 +1211,10 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             const int32_t* block_table, int table_width, int page_size,
                             int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
-                            int leave_splits, hipStream_t stream) {
+                            int leave_splits, int keep_first, float softcap, hipStream_t stream) {
   return launch_attn_mfma(q, q_stride, out, k_cache, v_cache, tiles, n_tiles, block_table, table_width, page_size,
                           head_dim, n_heads, n_kv, scale, window, n_waves, n_splits, workspace, workspace_floats,
-                          leave_splits, nullptr, false, stream);
+                          leave_splits, nullptr, false, stream, keep_first, softcap);
 }
 
 // yk_attn_mfma for a step of single tokens (every tile holds ONE token), with rotary + append

@@ -121,11 +121,11 @@ _SIGNATURES = {
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_attn_mfma_prefill": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp],
         _c_int,
     ),
     "yk_attn_mfma": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp],
         _c_int,
     ),
     "yk_attn_mfma_rope": (
@@ -848,7 +848,8 @@ class HipOps:
 
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
                   scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None,
-                  long_col_tiles: int = 1, token_cols=None, rope: Optional["RopeInLaunch"] = None):
+                  long_col_tiles: int = 1, token_cols=None, rope: Optional["RopeInLaunch"] = None,
+                  keep_first: int = 0, softcap: float = 0.0):
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
         block table of ``group``.  ``long_tiles`` hold up to
@@ -880,6 +881,8 @@ class HipOps:
             and qkv.stride(0) % 8 == 0
             and qkv.data_ptr() % 16 == 0
         )
+        if (keep_first or softcap) and not use_mfma:
+            raise KernelError("attention: kept first keys and squashed scores outside the matrix-core kernels' sizes are attention_masked's")
         if use_mfma and long_tiles is not None and long_tiles.shape[0] > 0:
             n_long = long_tiles.shape[0]
             hpt = self._ask("yk_attn_heads_per_tile", n_heads, n_kv)
@@ -892,7 +895,7 @@ class HipOps:
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     long_tiles.data_ptr(), n_long, bt.data_ptr(), bt.shape[1], page_size, head_dim,
                     n_heads, n_kv, float(scale), int(window), long_splits, int(long_col_tiles), _ptr(ws),
-                    0 if ws is None else ws.numel(), int(self.long_span_pages_in_lds),
+                    0 if ws is None else ws.numel(), int(self.long_span_pages_in_lds), int(keep_first), float(softcap),
                     self._stream(),
                 )
             )
@@ -912,7 +915,7 @@ class HipOps:
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     tiles.data_ptr(), n_tiles, bt.data_ptr(), bt.shape[1], page_size, head_dim, n_heads, n_kv,
                     float(scale), int(window), waves, splits, _ptr(ws), 0 if ws is None else ws.numel(), int(leave),
-                    self._stream(),
+                    int(keep_first), float(softcap), self._stream(),
                 )
             )
             if leave:

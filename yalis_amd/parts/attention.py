@@ -91,14 +91,16 @@ class Attention(Mixer):
             self.w_qkv = self.w_q = self.w_o = None
             self.b_qkv = self.b_q = self.b_o = None
             self.rotates_in_launch = False
+            # the matrix-core kernels take these options too, where they take the sizes (bfloat16, keys and
+            # values of 64 or 128 elements alike); everything else runs on the general float32-arithmetic kernel
+            can = getattr(rt.ops, "attention_can_rotate", None)
+            self.on_matrix_cores = bool(can is not None and self.value_dim == self.head_dim and can(rt.act_dtype, self.head_dim) is True)
+            if self.on_matrix_cores:
+                self._tile_sizes(rt)
             return
         rt.ops.check_attention_sizes(self.n_heads, self.n_kv, self.head_dim, rt.page_size)
-        self.tokens_per_tile = rt.ops.attention_tokens_per_tile(self.n_heads, self.n_kv)
-        # spans longer than `long_tile` go to the kernel for long spans, in tiles of that many
-        # tokens or twice as many (`long_tiles_of`: the step's choice)
-        self.long_tile = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
-        self.long_tile_2 = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv, 2)
-        self.layout = f"h{self.n_heads}g{self.n_kv}"
+        self.on_matrix_cores = True  # (where the kernel library has them for these sizes: it decides per call)
+        self._tile_sizes(rt)
         self.group = None
         self.w_qkv = self.w_q = self.w_o = None
         # whether the kernel library's attention can rotate and append inside its own launch
@@ -108,6 +110,14 @@ class Attention(Mixer):
         if self.rotates_in_launch:
             self.rope_in_launch = {append: rt.ops.rope_in_launch(self.rotation, append) for append in (False, True)}
         self.b_qkv = self.b_q = self.b_o = None
+
+    def _tile_sizes(self, rt) -> None:
+        self.tokens_per_tile = rt.ops.attention_tokens_per_tile(self.n_heads, self.n_kv)
+        # spans longer than `long_tile` go to the kernel for long spans, in tiles of that many
+        # tokens or twice as many (`long_tiles_of`: the step's choice)
+        self.long_tile = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
+        self.long_tile_2 = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv, 2)
+        self.layout = f"h{self.n_heads}g{self.n_kv}"
 
     # ---- what it needs
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -196,7 +206,7 @@ class Attention(Mixer):
         return self.rt.ops.attention_long_col_tiles(tiles * self.n_kv * chunks, fewest)
 
     def step_inputs(self):
-        if self.masked:
+        if self.masked and not self.on_matrix_cores:
             return {}
         # spans of more than one large tile go to the kernel for long spans, the rest
         # (single decoded tokens, short portions) to the one that splits the keys
@@ -230,6 +240,22 @@ class Attention(Mixer):
             page_size=self.rt.page_size,
         )
         gate_col = self.n_heads * self.head_dim + n_kv_rows * (self.head_dim + self.value_dim)
+        if self.on_matrix_cores:
+            memo_key = f"attention_long_col_tiles_{self.layout}"
+            col_tiles = ctx.memo.get(memo_key)
+            if col_tiles is None:
+                col_tiles = ctx.memo[memo_key] = self.long_col_tiles(ctx.host)
+            out = ops.attention(
+                q, self.n_heads, self.n_kv, self.head_dim, k_cache, v_cache, self.rt.page_size, self.scale,
+                0 if self.window is None else int(self.window), ctx, site.group,
+                ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"],
+                ctx.arrays[f"attention_long_tiles_{self.long_tile_2 if col_tiles == 2 else self.long_tile}_{self.layout}"],
+                long_col_tiles=col_tiles, keep_first=self.keep_first if self.window else 0, softcap=self.softcap,
+            )
+            if self.value_rotation is not None or self.gate_name:
+                ops.attention_finish(out, ctx.arrays["positions"], self.n_heads, self.value_dim, self.value_rotation,
+                                     gate=proj if self.gate_name else None, gate_col=gate_col)
+            return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
         out = ops.attention_masked(
             q, self.n_heads, self.n_kv, self.head_dim, self.value_dim, k_cache, v_cache, self.rt.page_size, self.scale, ctx,
             site.group, window=0 if self.window is None else int(self.window), keep_first=self.keep_first,
