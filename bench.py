@@ -518,6 +518,8 @@ def design_compare(args) -> int:
     from yalis_amd.models.presets import llama_like
 
     sizes = {"suranex": ("suranex-2k", "suranex-4k")}[args.design]
+    if args.design_shape:
+        sizes = (args.design_shape,)
     for name in sizes:
         label, cfg = SHAPES[name]
         line = {"design": args.design, "shape": label, "batch": args.batch, "prompt_len": args.prompt_len, "prefill_len": args.prefill_len,
@@ -546,6 +548,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--design", choices=("suranex",), default=None,
                     help="measure instead another design's prefill and decode at a few layer sizes, beside the Llama configuration of equal size, with the time and the bound of every kind of kernel")
+    ap.add_argument("--design-shape", default=None, help="with --design: one of its shapes only (suranex-2k, suranex-4k)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=32)
     ap.add_argument("--warmup", type=int, default=4)

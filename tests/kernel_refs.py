@@ -379,7 +379,7 @@ def causal_conv(x, weight, bias, state, ctx):
     return out.to(x.dtype)
 
 
-def rglru(u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx):
+def rglru(u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx, wa=None, wi=None, chunks=None, seq_chunk0=None):
     n, channels = u.shape
     blocks = wa_t.shape[0]
     a = ctx.arrays

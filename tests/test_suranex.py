@@ -108,6 +108,23 @@ def test_long_decoding(backend):
     assert held[0] >= 0 and held[1] < 0 and held[-1] >= 0 and sum(p >= 0 for p in held) <= 4
 
 
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["mix", "wide"])
+def test_long_prompt_in_one_step(backend, name):
+    """A prompt of 450 tokens whole, then a few tokens one by one: a span of many scan chunks, experts
+    with more than a hundred pairs each (the largest tiles), attention tiles far from the start."""
+    device, dtype = backend
+    if device == "cpu" and name == "wide":
+        pytest.skip("the plain ops are slow at this size; the GPU runs it")
+    cfg = X.CONFIGS[name]
+    weights = X.random_weights(cfg, seed=31)
+    reqs = X.make_requests(cfg, [456], seed=8)
+    want = X.plain_logits(cfg, weights, reqs)
+    runner = X.make_runner(cfg, weights, dtype, device, ops_for(device), X.PAGE[name], 16, max_seqs=1)
+    got, _ = C.run_trace(runner, C.trace_tail(reqs, tail=6))
+    X.assert_matches(got, want, dtype == "bfloat16", f"{name}/long prompt")
+
+
 def _one_layer(layer, mlp):
     return X.model(80, 32, 1e-5, [(layer, mlp)])
 

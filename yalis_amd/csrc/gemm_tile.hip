@@ -53,10 +53,24 @@ struct TilePlan {
   int m_tiles, n_tiles, splits, k_block;
 };
 
-template <typename TO>
+// The grouped form: a row block of x is a tile of a list made on the device (rows of (matrix,
+// first row, count <= 128) over rows that were sorted by the matrix they meet, `n_tiles` of them),
+// every tile multiplies its own matrix w + matrix * w_matrix_elems; sorted row i is row
+// x_rows[i] / x_div of x (x_rows null: row i) and its result is row y_rows[i] of y (null: row i).
+// A mixture of experts runs its two products through it.
+struct TileGroups {
+  const int32_t* tiles;
+  const int32_t* n_tiles;
+  const int32_t* x_rows;
+  int x_div;
+  const int32_t* y_rows;
+  size_t w_matrix_elems;
+};
+
+template <typename TO, bool GROUPED = false>
 __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part, TO* __restrict__ y,
-    int M, int N, int K, int ldx, int ldw, int ldy, TilePlan plan) {
+    int M, int N, int K, int ldx, int ldw, int ldy, TilePlan plan, TileGroups grp = TileGroups{}) {
   extern __shared__ __attribute__((aligned(16))) bf16_t lds_raw[];
   bf16_t(*lds)[GT_ROW] = reinterpret_cast<bf16_t(*)[GT_ROW]>(lds_raw);  // two buffers of [GT_BN + GT_BM][GT_ROW]
   const int lane = threadIdx.x % 64;
@@ -66,7 +80,14 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(
   const int die = blockIdx.x % GT_DIES, j = blockIdx.x / GT_DIES;
   const int n_tile = (j / plan.m_tiles) * GT_DIES + die, m_tile = j % plan.m_tiles;
   if (n_tile >= plan.n_tiles) return;  // (the grid is padded to whole groups of eight)
-  const int n0 = n_tile * GT_BN, m0 = m_tile * GT_BM;
+  int first = 0;  // GROUPED: the tile's first sorted row
+  if (GROUPED) {
+    if (m_tile >= *grp.n_tiles) return;
+    w += static_cast<size_t>(grp.tiles[3 * m_tile]) * grp.w_matrix_elems;
+    first = grp.tiles[3 * m_tile + 1];
+    M = grp.tiles[3 * m_tile + 2];  // the rows of this tile are all there is of x for it
+  }
+  const int n0 = n_tile * GT_BN, m0 = GROUPED ? 0 : m_tile * GT_BM;
   const int kb0 = blockIdx.y * plan.k_block;
   const int kb1 = min(K, kb0 + plan.k_block);
   const int wn = wave % 2, wm = wave / 2;
@@ -88,7 +109,9 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(
   for (int p = 0; p < GT_PIECES; ++p) {
     wsrc[p] = w + static_cast<size_t>(min(n0 + prow + 32 * p, N - 1)) * ldw;
     x_in[p] = m0 + prow + 32 * p < M;
-    xsrc[p] = x + static_cast<size_t>(min(m0 + prow + 32 * p, M - 1)) * ldx;
+    const int xi = min(m0 + prow + 32 * p, M - 1);
+    const int xrow = !GROUPED ? xi : (grp.x_rows ? grp.x_rows[first + xi] / grp.x_div : first + xi);
+    xsrc[p] = x + static_cast<size_t>(xrow) * ldx;
   }
   const int k_last = K - 8;
   const u32x4_t zero = {0u, 0u, 0u, 0u};
@@ -168,8 +191,9 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(
   const bool vec = pout ? N % 4 == 0 : (ldy % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0);
 #pragma unroll
   for (int jj = 0; jj < 2; ++jj) {
-    const int m = m0 + 64 * wm + 32 * jj + c;
+    int m = m0 + 64 * wm + 32 * jj + c;
     if (m >= M) continue;
+    if (GROUPED) m = grp.y_rows ? grp.y_rows[first + m] : first + m;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -239,7 +263,51 @@ int launch_tile(const bf16_t* x, const bf16_t* w, float* part, TO* y, int M, int
   return yk_check_launch("gemm_tile");
 }
 
+template <typename TO>
+int launch_tile_grouped(const bf16_t* x, const bf16_t* w, TO* y, int N, int K, int ldx, int ldw, int ldy, int max_tiles,
+                        const TileGroups& grp, hipStream_t stream) {
+  TilePlan plan;
+  plan.m_tiles = max_tiles;
+  plan.n_tiles = (N + GT_BN - 1) / GT_BN;
+  plan.splits = 1;
+  plan.k_block = (K + GT_BK - 1) / GT_BK * GT_BK;
+  const int groups = (plan.n_tiles + GT_DIES - 1) / GT_DIES;
+  dim3 grid(groups * plan.m_tiles * GT_DIES, 1);
+  constexpr size_t lds_bytes = 2 * static_cast<size_t>(GT_BN + GT_BM) * GT_ROW * sizeof(bf16_t);
+  static bool raised = false;
+  if (!raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<TO, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024) != hipSuccess)
+      return yk_fail("gemm_tile_grouped: cannot raise the LDS limit");
+    raised = true;
+  }
+  gemm_tile_kernel<TO, true><<<grid, dim3(256), lds_bytes, stream>>>(x, w, nullptr, y, 0, N, K, ldx, ldw, ldy, plan, grp);
+  return yk_check_launch("gemm_tile_grouped");
+}
+
 }  // namespace
+
+// The grouped form (see TileGroups): y[y_rows[i]] = x[x_rows[i] / x_div] . w[matrix of i]^T for the sorted
+// rows i of the tiles; `max_tiles` bounds the list's length (the launch has that many row blocks).
+extern "C" int yk_gemm_tile_grouped(const void* x, int ldx, const int32_t* x_rows, int x_div, const void* w,
+                                    size_t w_matrix_elems, int ldw, void* y, int y_dtype, int ldy, const int32_t* y_rows,
+                                    const int32_t* tiles, const int32_t* n_tiles, int max_tiles, int N, int K,
+                                    hipStream_t stream) {
+  YK_REQUIRE(max_tiles >= 0 && N > 0 && K >= 8, "gemm_tile_grouped: bad sizes");
+  YK_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && w_matrix_elems % 8 == 0,
+             "gemm_tile_grouped: K and the leading dimensions must be multiples of 8");
+  YK_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
+             "gemm_tile_grouped: operands must be 16-byte aligned");
+  YK_REQUIRE(ldx >= K && ldw >= K && ldy >= N && x_div >= 1, "gemm_tile_grouped: leading dimensions too small");
+  YK_REQUIRE(y_dtype == YK_F32 || y_dtype == YK_BF16, "gemm_tile_grouped: unsupported output dtype");
+  YK_REQUIRE(static_cast<long>(max_tiles) * (((N + GT_BN - 1) / GT_BN + 7) / 8) * 8 <= 0x7fffffffL / 2, "gemm_tile_grouped: too many tiles");
+  if (max_tiles == 0) return 0;
+  TileGroups grp{tiles, n_tiles, x_rows, x_div, y_rows, w_matrix_elems};
+  const bf16_t* xp = static_cast<const bf16_t*>(x);
+  const bf16_t* wp = static_cast<const bf16_t*>(w);
+  if (y_dtype == YK_F32) return launch_tile_grouped<float>(xp, wp, static_cast<float*>(y), N, K, ldx, ldw, ldy, max_tiles, grp, stream);
+  return launch_tile_grouped<bf16_t>(xp, wp, static_cast<bf16_t*>(y), N, K, ldx, ldw, ldy, max_tiles, grp, stream);
+}
 
 // For tests and measurements: force the number of K slices (0: the library decides).
 extern "C" int yk_gemm_tile_force(int splits) {

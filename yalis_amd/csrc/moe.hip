@@ -13,7 +13,7 @@
 //   * moe_down: rows[pair, :] = y[i, :] . Wd_e^T in float32, stored in pair order (token-major), so
 //     that whoever adds a token's rows finds them side by side (the norm that follows does).
 // Each product has a float32 FMA form for any sizes and dtypes, and a matrix-core form for
-// bfloat16 with K a multiple of 32: a wave multiplies 16 weight rows (the A operand, straight
+// bfloat16 with K a multiple of 32: a wave multiplies 16 * FT weight rows (the A operand, straight
 // from memory) with 16 * MT pairs (the B operand, gathered rows of x), so an expert's weights are
 // read once per tile of pairs.
 #include <algorithm>
@@ -144,83 +144,150 @@ union MoeFrag {
 // Operands of v_mfma_f32_16x16x32_bf16 (r = lane % 16, g = lane / 16): A lane holds A[r][8g..8g+7],
 // B lane holds B[8g..8g+7][r], C lane holds C[4g..4g+3][r].  A = 16 weight rows, B = 16 pairs'
 // rows of x: C[i][r] = (pair r, feature 4g + i).
-template <int MT>
-__global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
+// A wave owns FT tiles of 16 features and MT tiles of 16 pairs; the fragments of the next step
+// of 32 along K are asked for before the products of this one are issued (two register sets by
+// turns), so that loads and matrix cores overlap.
+//
+// A workgroup has 4 * WR waves: four side by side over the features, WR one above the other over
+// the tile's pairs (16 * MT each).  Workgroups are numbered so that those that share a tile's pairs
+// (one per group of features) come one behind the other on one die (numbers 8 apart), whose L2 then
+// holds the tile's rows of x for all of them; every weight row is read once per tile.
+__device__ __forceinline__ void moe_tile_of(int n_groups, int& tile, int& group) {
+  const int die = blockIdx.x % 8, slot = blockIdx.x / 8;
+  tile = (slot / n_groups) * 8 + die;
+  group = slot % n_groups;
+}
+
+template <int MT, int FT, int WR>
+__global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
     const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, int top, int hidden, int ff, int kind,
-    float p0, float p1, bf16_t* __restrict__ y) {
-  const int t = blockIdx.x;
+    float p0, float p1, bf16_t* __restrict__ y, int n_groups) {
+  int t, group;
+  moe_tile_of(n_groups, t, group);
   if (t >= *n_tiles) return;
-  const int e = tiles[3 * t], first = tiles[3 * t + 1], count = tiles[3 * t + 2];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r = lane % 16, g = lane / 16;
-  const int f0 = (blockIdx.y * 4 + wave) * 16;
-  if (f0 >= ff) return;
-  const bf16_t* wg = w + (static_cast<size_t>(e) * 2 * ff + f0 + r) * hidden + 8 * g;
-  const bf16_t* wu = wg + static_cast<size_t>(ff) * hidden;
+  const int e = tiles[3 * t], row0 = 16 * MT * (wave / 4);
+  const int first = tiles[3 * t + 1] + row0, count = tiles[3 * t + 2] - row0;
+  const int f0 = (group * 4 + wave % 4) * 16 * FT;
+  if (f0 >= ff || count <= 0) return;
+  const bf16_t *wg[FT], *wu[FT];
+#pragma unroll
+  for (int f = 0; f < FT; ++f) {
+    const int row = min(f0 + 16 * f + r, ff - 1);  // (tiles beyond the width repeat its last row and are not stored)
+    wg[f] = w + (static_cast<size_t>(e) * 2 * ff + row) * hidden + 8 * g;
+    wu[f] = wg[f] + static_cast<size_t>(ff) * hidden;
+  }
   const bf16_t* xr[MT];
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     const int slot = first + min(16 * m + r, count - 1);  // rows beyond the tile repeat its last pair and are not stored
     xr[m] = x + static_cast<size_t>(order[slot] / top) * x_stride + 8 * g;
   }
-  f32x4_t ag[MT], au[MT];
+  f32x4_t ag[FT][MT], au[FT][MT];
 #pragma unroll
-  for (int m = 0; m < MT; ++m) ag[m] = au[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < hidden; k0 += 32) {
-    MoeFrag a_g, a_u, b[MT];
-    a_g.u = *reinterpret_cast<const u32x4_t*>(wg + k0);
-    a_u.u = *reinterpret_cast<const u32x4_t*>(wu + k0);
+  for (int f = 0; f < FT; ++f)
 #pragma unroll
-    for (int m = 0; m < MT; ++m) b[m].u = *reinterpret_cast<const u32x4_t*>(xr[m] + k0);
+    for (int m = 0; m < MT; ++m) ag[f][m] = au[f][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  MoeFrag a0[2][FT], b0[MT], a1[2][FT], b1[MT];
+#define MOE_LOAD(A, B, K0)                                                                  \
+  {                                                                                         \
+    _Pragma("unroll") for (int f = 0; f < FT; ++f) {                                        \
+      A[0][f].u = *reinterpret_cast<const u32x4_t*>(wg[f] + (K0));                          \
+      A[1][f].u = *reinterpret_cast<const u32x4_t*>(wu[f] + (K0));                          \
+    }                                                                                       \
+    _Pragma("unroll") for (int m = 0; m < MT; ++m) B[m].u = *reinterpret_cast<const u32x4_t*>(xr[m] + (K0)); \
+  }
+#define MOE_MMA(A, B)                                                                       \
+  {                                                                                         \
+    _Pragma("unroll") for (int f = 0; f < FT; ++f)                                          \
+    _Pragma("unroll") for (int m = 0; m < MT; ++m) {                                        \
+      ag[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[0][f].v, B[m].v, ag[f][m], 0, 0, 0); \
+      au[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[1][f].v, B[m].v, au[f][m], 0, 0, 0); \
+    }                                                                                       \
+  }
+  MOE_LOAD(a0, b0, 0)
+  for (int k0 = 0; k0 < hidden; k0 += 64) {
+    const bool second = k0 + 32 < hidden;
+    if (second) MOE_LOAD(a1, b1, k0 + 32)
+    MOE_MMA(a0, b0)
+    if (k0 + 64 < hidden) MOE_LOAD(a0, b0, k0 + 64)
+    if (second) MOE_MMA(a1, b1)
+  }
+#undef MOE_LOAD
+#undef MOE_MMA
+#pragma unroll
+  for (int f = 0; f < FT; ++f) {
+    if (f0 + 16 * f >= ff) continue;
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-      ag[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_g.v, b[m].v, ag[m], 0, 0, 0);
-      au[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_u.v, b[m].v, au[m], 0, 0, 0);
-    }
-  }
-#pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    if (16 * m + r < count) {
-      uint32_t o[2];
-      o[0] = pack_bf16x2(gated_pair(ag[m][0], au[m][0], kind, p0, p1), gated_pair(ag[m][1], au[m][1], kind, p0, p1));
-      o[1] = pack_bf16x2(gated_pair(ag[m][2], au[m][2], kind, p0, p1), gated_pair(ag[m][3], au[m][3], kind, p0, p1));
-      *reinterpret_cast<uint2*>(y + static_cast<size_t>(first + 16 * m + r) * ff + f0 + 4 * g) = make_uint2(o[0], o[1]);
+      if (16 * m + r < count) {
+        uint32_t o[2];
+        o[0] = pack_bf16x2(gated_pair(ag[f][m][0], au[f][m][0], kind, p0, p1), gated_pair(ag[f][m][1], au[f][m][1], kind, p0, p1));
+        o[1] = pack_bf16x2(gated_pair(ag[f][m][2], au[f][m][2], kind, p0, p1), gated_pair(ag[f][m][3], au[f][m][3], kind, p0, p1));
+        *reinterpret_cast<uint2*>(y + static_cast<size_t>(first + 16 * m + r) * ff + f0 + 16 * f + 4 * g) = make_uint2(o[0], o[1]);
+      }
     }
   }
 }
 
-template <int MT>
-__global__ __launch_bounds__(256) void moe_down_mfma_kernel(
+template <int MT, int FT, int WR>
+__global__ __launch_bounds__(256 * WR) void moe_down_mfma_kernel(
     const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, int hidden, int ff,
-    float* __restrict__ rows) {
-  const int t = blockIdx.x;
+    float* __restrict__ rows, int n_groups) {
+  int t, group;
+  moe_tile_of(n_groups, t, group);
   if (t >= *n_tiles) return;
-  const int e = tiles[3 * t], first = tiles[3 * t + 1], count = tiles[3 * t + 2];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r = lane % 16, g = lane / 16;
-  const int h0 = (blockIdx.y * 4 + wave) * 16;
-  if (h0 >= hidden) return;
-  const bf16_t* wd = w + (static_cast<size_t>(e) * hidden + h0 + r) * ff + 8 * g;
+  const int e = tiles[3 * t], row0 = 16 * MT * (wave / 4);
+  const int first = tiles[3 * t + 1] + row0, count = tiles[3 * t + 2] - row0;
+  const int h0 = (group * 4 + wave % 4) * 16 * FT;
+  if (h0 >= hidden || count <= 0) return;
+  const bf16_t* wd[FT];
+#pragma unroll
+  for (int f = 0; f < FT; ++f)
+    wd[f] = w + (static_cast<size_t>(e) * hidden + min(h0 + 16 * f + r, hidden - 1)) * ff + 8 * g;
   const bf16_t* yr[MT];
 #pragma unroll
   for (int m = 0; m < MT; ++m) yr[m] = y + static_cast<size_t>(first + min(16 * m + r, count - 1)) * ff + 8 * g;
-  f32x4_t acc[MT];
+  f32x4_t acc[FT][MT];
 #pragma unroll
-  for (int m = 0; m < MT; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < ff; k0 += 32) {
-    MoeFrag a, b[MT];
-    a.u = *reinterpret_cast<const u32x4_t*>(wd + k0);
+  for (int f = 0; f < FT; ++f)
 #pragma unroll
-    for (int m = 0; m < MT; ++m) b[m].u = *reinterpret_cast<const u32x4_t*>(yr[m] + k0);
-#pragma unroll
-    for (int m = 0; m < MT; ++m) acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[m].v, acc[m], 0, 0, 0);
+    for (int m = 0; m < MT; ++m) acc[f][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  MoeFrag a0[FT], b0[MT], a1[FT], b1[MT];
+#define MOE_LOAD(A, B, K0)                                                                  \
+  {                                                                                         \
+    _Pragma("unroll") for (int f = 0; f < FT; ++f) A[f].u = *reinterpret_cast<const u32x4_t*>(wd[f] + (K0)); \
+    _Pragma("unroll") for (int m = 0; m < MT; ++m) B[m].u = *reinterpret_cast<const u32x4_t*>(yr[m] + (K0)); \
   }
+#define MOE_MMA(A, B)                                                                       \
+  {                                                                                         \
+    _Pragma("unroll") for (int f = 0; f < FT; ++f)                                          \
+    _Pragma("unroll") for (int m = 0; m < MT; ++m)                                          \
+      acc[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[f].v, B[m].v, acc[f][m], 0, 0, 0); \
+  }
+  MOE_LOAD(a0, b0, 0)
+  for (int k0 = 0; k0 < ff; k0 += 64) {
+    const bool second = k0 + 32 < ff;
+    if (second) MOE_LOAD(a1, b1, k0 + 32)
+    MOE_MMA(a0, b0)
+    if (k0 + 64 < ff) MOE_LOAD(a0, b0, k0 + 64)
+    if (second) MOE_MMA(a1, b1)
+  }
+#undef MOE_LOAD
+#undef MOE_MMA
 #pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    if (16 * m + r < count) {
-      const int pair = order[first + 16 * m + r];
-      *reinterpret_cast<float4*>(rows + static_cast<size_t>(pair) * hidden + h0 + 4 * g) =
-          make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+  for (int f = 0; f < FT; ++f) {
+    if (h0 + 16 * f >= hidden) continue;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      if (16 * m + r < count) {
+        const int pair = order[first + 16 * m + r];
+        *reinterpret_cast<float4*>(rows + static_cast<size_t>(pair) * hidden + h0 + 16 * f + 4 * g) =
+            make_float4(acc[f][m][0], acc[f][m][1], acc[f][m][2], acc[f][m][3]);
+      }
     }
   }
 }
@@ -240,14 +307,20 @@ extern "C" int yk_moe_gate_up(const void* x, int x_stride, int dtype, const void
   YK_REQUIRE(kind >= 0 && kind < YK_GATED_KINDS, "moe_gate_up: unknown activation");
   if (n_pairs == 0) return 0;
   if (dtype == YK_BF16 && w_dtype == YK_BF16 && yk_moe_mfma_ok(hidden, ff, x_stride) && aligned16(x) && aligned16(w) &&
-      aligned16(y) && (tile_rows == 16 || tile_rows == 64)) {
-    dim3 grid(max_tiles, (ff + 63) / 64), block(256);
-    if (tile_rows == 16)
-      moe_gate_up_mfma_kernel<1><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w),
-                                                            order, tiles, n_tiles, top, hidden, ff, kind, p0, p1, static_cast<bf16_t*>(y));
-    else
-      moe_gate_up_mfma_kernel<4><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w),
-                                                            order, tiles, n_tiles, top, hidden, ff, kind, p0, p1, static_cast<bf16_t*>(y));
+      aligned16(y) && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128)) {
+    constexpr int FT = 2;  // feature tiles of 16 a wave
+    const int n_groups = (ff + 64 * FT - 1) / (64 * FT);
+    const long long n_wg = static_cast<long long>((max_tiles + 7) / 8 * 8) * n_groups;
+    YK_REQUIRE(n_wg <= 0x7fffffffLL, "moe_gate_up: too many tiles for one launch");
+    dim3 grid(static_cast<unsigned>(n_wg));
+#define YK_MOE_GU(MT, WR)                                                                                       \
+  moe_gate_up_mfma_kernel<MT, FT, WR><<<grid, 256 * WR, 0, stream>>>(                                            \
+      static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w), order, tiles, n_tiles, top, hidden, ff, \
+      kind, p0, p1, static_cast<bf16_t*>(y), n_groups)
+    if (tile_rows == 16) YK_MOE_GU(1, 1);
+    else if (tile_rows == 64) YK_MOE_GU(4, 1);
+    else YK_MOE_GU(4, 2);
+#undef YK_MOE_GU
     return yk_check_launch("moe_gate_up (matrix cores)");
   }
   YK_REQUIRE(hidden <= 15 * 1024, "moe_gate_up: rows of more than 15,360 elements do not fit");
@@ -273,14 +346,19 @@ extern "C" int yk_moe_down(const void* y, int dtype, const void* w, int w_dtype,
   YK_REQUIRE(n_pairs >= 0 && hidden > 0 && ff > 0, "moe_down: bad sizes");
   if (n_pairs == 0) return 0;
   if (dtype == YK_BF16 && w_dtype == YK_BF16 && yk_moe_mfma_ok(ff, hidden, ff) && aligned16(y) && aligned16(w) &&
-      aligned16(rows) && (tile_rows == 16 || tile_rows == 64)) {
-    dim3 grid(max_tiles, (hidden + 63) / 64), block(256);
-    if (tile_rows == 16)
-      moe_down_mfma_kernel<1><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(y), static_cast<const bf16_t*>(w), order,
-                                                         tiles, n_tiles, hidden, ff, rows);
-    else
-      moe_down_mfma_kernel<4><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(y), static_cast<const bf16_t*>(w), order,
-                                                         tiles, n_tiles, hidden, ff, rows);
+      aligned16(rows) && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128)) {
+    constexpr int FT = 4;
+    const int n_groups = (hidden + 64 * FT - 1) / (64 * FT);
+    const long long n_wg = static_cast<long long>((max_tiles + 7) / 8 * 8) * n_groups;
+    YK_REQUIRE(n_wg <= 0x7fffffffLL, "moe_down: too many tiles for one launch");
+    dim3 grid(static_cast<unsigned>(n_wg));
+#define YK_MOE_DN(MT, WR)                                                                                       \
+  moe_down_mfma_kernel<MT, FT, WR><<<grid, 256 * WR, 0, stream>>>(static_cast<const bf16_t*>(y), static_cast<const bf16_t*>(w), \
+                                                                  order, tiles, n_tiles, hidden, ff, rows, n_groups)
+    if (tile_rows == 16) YK_MOE_DN(1, 1);
+    else if (tile_rows == 64) YK_MOE_DN(4, 1);
+    else YK_MOE_DN(4, 2);
+#undef YK_MOE_DN
     return yk_check_launch("moe_down (matrix cores)");
   }
   YK_REQUIRE(ff <= 15 * 1024, "moe_down: rows of more than 15,360 elements do not fit");

@@ -185,3 +185,23 @@ def attention_token_columns(hb: HostBatch, tokens_per_tile: int, min_span: int =
             tile += 1
     return cols
 
+
+
+def span_chunks(hb: HostBatch, chunk: int) -> np.ndarray:
+    """Every request's span cut into chunks of at most ``chunk`` consecutive tokens, in the order of
+    the requests: rows of (request, first token index in the batch, token count).  A scan over a
+    span can then run chunk by chunk (``chunk_starts`` says which rows are whose)."""
+    rows = []
+    for i in range(hb.n_seqs):
+        q0, ql = int(hb.seq_qstart[i]), int(hb.seq_qlen[i])
+        for t in range(0, ql, chunk):
+            rows.append((i, q0 + t, min(chunk, ql - t)))
+    return np.array(rows, dtype=np.int32).reshape(-1, 3)
+
+
+def chunk_starts(hb: HostBatch, chunk: int) -> np.ndarray:
+    """[requests + 1]: the first row of ``span_chunks`` of every request, and the number of rows."""
+    counts = -(-hb.seq_qlen.astype(np.int64) // chunk)
+    out = np.zeros(hb.n_seqs + 1, dtype=np.int32)
+    np.cumsum(counts, out=out[1:])
+    return out

@@ -81,7 +81,12 @@ _SIGNATURES = {
         _c_int,
     ),
     "yk_causal_conv": ([_vp, _c_int, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
-    "yk_rglru_gates": ([_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_rglru_gates": ([_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _vp], _c_int),
+    "yk_rglru_gates_mfma_ok": ([_c_int, _c_int], _c_int),
+    "yk_rglru_scan_chunked": (
+        [_vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
     "yk_rglru_scan": ([_vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_moe_max_tiles": ([_c_int, _c_int, _c_int], _c_int),
     "yk_moe_mfma_ok": ([_c_int, _c_int, _c_int], _c_int),
@@ -110,6 +115,10 @@ _SIGNATURES = {
         _c_int,
     ),
     "yk_gemm_tile_splits": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_tile_grouped": (
+        [_vp, _c_int, _vp, _c_int, _vp, _c_size_t, _c_int, _vp, _c_int, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
     "yk_gemm_tile_force": ([_c_int], _c_int),
     "yk_attn_generic": (
         [_vp, _c_int, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
@@ -1218,11 +1227,18 @@ class HipOps:
         )
         return out
 
-    def rglru(self, u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx) -> torch.Tensor:
+    # spans of more than this many tokens are scanned in chunks (cut by the caller)
+    RGLRU_CHUNKED_FROM = 32
+
+    def rglru(self, u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx, wa=None, wi=None,
+              chunks=None, seq_chunk0=None) -> torch.Tensor:
         """The real-gated linear recurrence over each request's span.  ``u`` [N, C] the convolved
         branch, ``y`` [N, C] the other branch before its gelu, ``x`` [N, C] the convolution's inputs (its
-        state is brought up to date here); gate matrices transposed [blocks, in, out].  Returns S_t *
-        gelu(y_t) [N, C]; ``s_state`` [slots, C] float32 and ``conv_state`` are left as after the span."""
+        state is brought up to date here); gate matrices transposed [blocks, in, out] (and, as ``wa`` /
+        ``wi``, in their own layout [blocks, out, in], which the matrix-core form of the gates reads).
+        ``chunks`` [n, 3] (request, first token, count) and ``seq_chunk0`` [requests + 1] cut the spans for
+        the scan in chunks, which runs when the step's longest span exceeds ``RGLRU_CHUNKED_FROM``.  Returns
+        S_t * gelu(y_t) [N, C]; ``s_state`` [slots, C] float32 and ``conv_state`` are left as after the span."""
         n, channels = u.shape
         blocks = wa_t.shape[0]
         bs = channels // blocks
@@ -1240,11 +1256,24 @@ class HipOps:
         self._check(
             self.lib.yk_rglru_gates(
                 u.data_ptr(), _code(u.dtype), wa_t.data_ptr(), ba.data_ptr(), wi_t.data_ptr(), bi.data_ptr(), lam.data_ptr(),
-                _code(wa_t.dtype), float(rate), a.data_ptr(), b.data_ptr(), n, channels, blocks, self._stream(),
+                _code(wa_t.dtype), float(rate), a.data_ptr(), b.data_ptr(), n, channels, blocks,
+                _ptr(wa) if wa is not None and wa.is_contiguous() and wa.dtype == wa_t.dtype else None,
+                _ptr(wi) if wi is not None and wi.is_contiguous() and wi.dtype == wa_t.dtype else None, self._stream(),
             )
         )
         out = torch.empty((n, channels), dtype=u.dtype, device=u.device)
         arr = ctx.arrays
+        if chunks is not None and ctx.max_qlen > self.RGLRU_CHUNKED_FROM:
+            pq = torch.empty((chunks.shape[0], 2, channels), dtype=torch.float32, device=u.device)
+            self._check(
+                self.lib.yk_rglru_scan_chunked(
+                    a.data_ptr(), b.data_ptr(), y.data_ptr(), y.stride(0), x.data_ptr(), x.stride(0), _code(u.dtype),
+                    s_state.data_ptr(), _ptr(conv_state), arr["seq_qstart"].data_ptr(), arr["seq_qlen"].data_ptr(),
+                    arr["state_slots"].data_ptr(), chunks.data_ptr(), chunks.shape[0], seq_chunk0.data_ptr(), pq.data_ptr(),
+                    out.data_ptr(), arr["seq_qstart"].numel(), channels, int(taps), self._stream(),
+                )
+            )
+            return out
         self._check(
             self.lib.yk_rglru_scan(
                 a.data_ptr(), b.data_ptr(), y.data_ptr(), y.stride(0), x.data_ptr(), x.stride(0), _code(u.dtype),
@@ -1273,8 +1302,8 @@ class HipOps:
         rows = torch.empty((pairs, hidden), dtype=torch.float32, device=dev)
         if n == 0:
             return rows
-        # tiles of 64 pairs where an expert has that many on average, else of 16
-        tile_rows = 64 if pairs >= 48 * experts else 16
+        # tiles of 128 or 64 pairs where an expert has that many on average, else of 16
+        tile_rows = 128 if pairs >= 96 * experts else (64 if pairs >= 48 * experts else 16)
         max_tiles = self.lib.yk_moe_max_tiles(pairs, experts, tile_rows)
         ints = torch.empty(2 * pairs + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
         order, slot_expert = ints[:pairs], ints[pairs: 2 * pairs]
@@ -1283,6 +1312,26 @@ class HipOps:
             self.lib.yk_moe_route(token_ids.data_ptr(), table.data_ptr(), vocab, top, experts, n, tile_rows, order.data_ptr(),
                                   slot_expert.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), self._stream())
         )
+        bf = torch.bfloat16
+        if (tile_rows == 128 and x.dtype == bf and w_gate_up.dtype == bf and w_down.dtype == bf and hidden % 8 == 0 and ff % 8 == 0
+                and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+            # many pairs an expert: both products as tiles of 128 x 128 through LDS (the grouped form of
+            # ``gemm_tile``), the gated pair by the activation kernel between them
+            gu = torch.empty((pairs, 2 * ff), dtype=bf, device=dev)
+            self._check(
+                self.lib.yk_gemm_tile_grouped(
+                    x.data_ptr(), x.stride(0), order.data_ptr(), top, w_gate_up.data_ptr(), 2 * ff * hidden, hidden, gu.data_ptr(),
+                    _BF16, 2 * ff, None, tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, 2 * ff, hidden, self._stream(),
+                )
+            )
+            y = self.gated_act(gu, activation, bf)
+            self._check(
+                self.lib.yk_gemm_tile_grouped(
+                    y.data_ptr(), ff, None, 1, w_down.data_ptr(), hidden * ff, ff, rows.data_ptr(), _F32, hidden,
+                    order.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, hidden, ff, self._stream(),
+                )
+            )
+            return rows
         y = torch.empty((pairs, ff), dtype=x.dtype, device=dev)
         self._check(
             self.lib.yk_moe_gate_up(

@@ -14,7 +14,8 @@ conv_taps - 1 inputs of the convolution; both live in the request's slot and sta
 Gates, decays and the recurrence are float32 in both engines.
 
 params: prefix, hidden_size, width, blocks, conv_taps, rate (8.0: the constant in front of
-r * softplus(lam)), names (optional overrides of the tensor names below the prefix).
+r * softplus(lam)), scan_chunk (64: tokens of a chunk when a long span is scanned in chunks), names
+(optional overrides of the tensor names below the prefix).
 """
 from __future__ import annotations
 
@@ -22,6 +23,7 @@ from typing import Dict, Mapping
 
 import torch
 
+from ..engine.batch import chunk_starts, span_chunks
 from ..weights.loader import TensorSpec
 from .base import Mixer, Runtime, StateNeed, register_mixer
 
@@ -48,6 +50,9 @@ class RecurrentGatedUnit(Mixer):
         self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
         self.w_yx = self.b_yx = self.w_conv = self.b_conv = self.w_o = None
         self.wa_t = self.wi_t = self.ba = self.bi = self.lam = None
+        self.wa = self.wi = None
+        # long spans are scanned in chunks of this many tokens
+        self.chunk = int(params.get("scan_chunk", 64))
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         c, bs, n = self.width, self.width // self.blocks, self.names
@@ -70,8 +75,9 @@ class RecurrentGatedUnit(Mixer):
         self.w_conv, self.b_conv = tensors[n["conv"]].contiguous(), tensors[n["conv_bias"]].contiguous()
         # gate matrices [block, out, in] are kept [block, in, out]: the kernel's threads, one per output
         # channel, then read consecutive addresses
-        self.wa_t = tensors[n["ra"]].transpose(1, 2).contiguous()
-        self.wi_t = tensors[n["ri"]].transpose(1, 2).contiguous()
+        self.wa, self.wi = tensors[n["ra"]].contiguous(), tensors[n["ri"]].contiguous()  # (what the matrix-core form reads)
+        self.wa_t = self.wa.transpose(1, 2).contiguous()
+        self.wi_t = self.wi.transpose(1, 2).contiguous()
         self.ba = tensors[n["ra_bias"]].reshape(-1).contiguous()
         self.bi = tensors[n["ri_bias"]].reshape(-1).contiguous()
         self.lam = tensors[n["lam"]].contiguous()
@@ -91,6 +97,10 @@ class RecurrentGatedUnit(Mixer):
     def products(self):
         return ((2 * self.width, self.hidden), (self.hidden, self.width))
 
+    def step_inputs(self):
+        n = self.chunk
+        return {f"span_chunks_{n}": lambda hb: span_chunks(hb, n), f"chunk_starts_{n}": lambda hb: chunk_starts(hb, n)}
+
     def forward(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
         ops = self.rt.ops
         yx = ops.linear(h, self.w_yx, self.rt.act_dtype, bias=self.b_yx)
@@ -98,5 +108,6 @@ class RecurrentGatedUnit(Mixer):
         conv_state = site.state(1) if self.taps > 1 else None
         u = ops.causal_conv(x, self.w_conv, self.b_conv, conv_state, ctx)
         s = ops.rglru(u, y, x, self.wa_t, self.ba, self.wi_t, self.bi, self.lam, self.rate, site.state(0), conv_state,
-                      self.taps, ctx)
+                      self.taps, ctx, wa=self.wa, wi=self.wi, chunks=ctx.arrays[f"span_chunks_{self.chunk}"],
+                      seq_chunk0=ctx.arrays[f"chunk_starts_{self.chunk}"])
         return ops.linear(s, self.w_o, self.rt.act_dtype, partial_ok=True)
