@@ -158,7 +158,10 @@ __device__ __forceinline__ void moe_tile_of(int n_groups, int& tile, int& group)
   group = slot % n_groups;
 }
 
-template <int MT, int FT, int WR>
+// KS: the four waves of a workgroup share one set of features and divide K between them (their
+// sums meet in LDS): steps of few pairs have few tiles, and this way four times the waves pull on
+// an expert's weights.
+template <int MT, int FT, int WR, bool KS>
 __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
     const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, int top, int hidden, int ff, int kind,
@@ -169,8 +172,10 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r = lane % 16, g = lane / 16;
   const int e = tiles[3 * t], row0 = 16 * MT * (wave / 4);
   const int first = tiles[3 * t + 1] + row0, count = tiles[3 * t + 2] - row0;
-  const int f0 = (group * 4 + wave % 4) * 16 * FT;
+  const int f0 = (KS ? group : group * 4 + wave % 4) * 16 * FT;
   if (f0 >= ff || count <= 0) return;
+  const int k_quarter = ((hidden / 32 + 3) / 4) * 32;
+  const int k_begin = KS ? wave * k_quarter : 0, k_end = KS ? min(hidden, k_begin + k_quarter) : hidden;
   const bf16_t *wg[FT], *wu[FT];
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
@@ -206,16 +211,39 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
       au[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[1][f].v, B[m].v, au[f][m], 0, 0, 0); \
     }                                                                                       \
   }
-  MOE_LOAD(a0, b0, 0)
-  for (int k0 = 0; k0 < hidden; k0 += 64) {
-    const bool second = k0 + 32 < hidden;
+  if (k_begin < k_end) MOE_LOAD(a0, b0, k_begin)
+  for (int k0 = k_begin; k0 < k_end; k0 += 64) {
+    const bool second = k0 + 32 < k_end;
     if (second) MOE_LOAD(a1, b1, k0 + 32)
     MOE_MMA(a0, b0)
-    if (k0 + 64 < hidden) MOE_LOAD(a0, b0, k0 + 64)
+    if (k0 + 64 < k_end) MOE_LOAD(a0, b0, k0 + 64)
     if (second) MOE_MMA(a1, b1)
   }
 #undef MOE_LOAD
 #undef MOE_MMA
+  if (KS) {
+    __shared__ f32x4_t part[3][2 * FT * MT][64];
+    if (wave > 0) {
+#pragma unroll
+      for (int f = 0; f < FT; ++f)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          part[wave - 1][(2 * f) * MT + m][lane] = ag[f][m];
+          part[wave - 1][(2 * f + 1) * MT + m][lane] = au[f][m];
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w2 = 0; w2 < 3; ++w2)
+#pragma unroll
+      for (int f = 0; f < FT; ++f)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          ag[f][m] += part[w2][(2 * f) * MT + m][lane];
+          au[f][m] += part[w2][(2 * f + 1) * MT + m][lane];
+        }
+  }
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
     if (f0 + 16 * f >= ff) continue;
@@ -231,7 +259,7 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
   }
 }
 
-template <int MT, int FT, int WR>
+template <int MT, int FT, int WR, bool KS>
 __global__ __launch_bounds__(256 * WR) void moe_down_mfma_kernel(
     const bf16_t* __restrict__ y, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, int hidden, int ff,
@@ -242,8 +270,10 @@ __global__ __launch_bounds__(256 * WR) void moe_down_mfma_kernel(
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, r = lane % 16, g = lane / 16;
   const int e = tiles[3 * t], row0 = 16 * MT * (wave / 4);
   const int first = tiles[3 * t + 1] + row0, count = tiles[3 * t + 2] - row0;
-  const int h0 = (group * 4 + wave % 4) * 16 * FT;
+  const int h0 = (KS ? group : group * 4 + wave % 4) * 16 * FT;
   if (h0 >= hidden || count <= 0) return;
+  const int k_quarter = ((ff / 32 + 3) / 4) * 32;
+  const int k_begin = KS ? wave * k_quarter : 0, k_end = KS ? min(ff, k_begin + k_quarter) : ff;
   const bf16_t* wd[FT];
 #pragma unroll
   for (int f = 0; f < FT; ++f)
@@ -268,16 +298,33 @@ __global__ __launch_bounds__(256 * WR) void moe_down_mfma_kernel(
     _Pragma("unroll") for (int m = 0; m < MT; ++m)                                          \
       acc[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[f].v, B[m].v, acc[f][m], 0, 0, 0); \
   }
-  MOE_LOAD(a0, b0, 0)
-  for (int k0 = 0; k0 < ff; k0 += 64) {
-    const bool second = k0 + 32 < ff;
+  if (k_begin < k_end) MOE_LOAD(a0, b0, k_begin)
+  for (int k0 = k_begin; k0 < k_end; k0 += 64) {
+    const bool second = k0 + 32 < k_end;
     if (second) MOE_LOAD(a1, b1, k0 + 32)
     MOE_MMA(a0, b0)
-    if (k0 + 64 < ff) MOE_LOAD(a0, b0, k0 + 64)
+    if (k0 + 64 < k_end) MOE_LOAD(a0, b0, k0 + 64)
     if (second) MOE_MMA(a1, b1)
   }
 #undef MOE_LOAD
 #undef MOE_MMA
+  if (KS) {
+    __shared__ f32x4_t part[3][FT * MT][64];
+    if (wave > 0) {
+#pragma unroll
+      for (int f = 0; f < FT; ++f)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) part[wave - 1][f * MT + m][lane] = acc[f][m];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w2 = 0; w2 < 3; ++w2)
+#pragma unroll
+      for (int f = 0; f < FT; ++f)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[f][m] += part[w2][f * MT + m][lane];
+  }
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
     if (h0 + 16 * f >= hidden) continue;
@@ -309,17 +356,17 @@ extern "C" int yk_moe_gate_up(const void* x, int x_stride, int dtype, const void
   if (dtype == YK_BF16 && w_dtype == YK_BF16 && yk_moe_mfma_ok(hidden, ff, x_stride) && aligned16(x) && aligned16(w) &&
       aligned16(y) && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128)) {
     constexpr int FT = 2;  // feature tiles of 16 a wave
-    const int n_groups = (ff + 64 * FT - 1) / (64 * FT);
+    const int n_groups = tile_rows == 16 ? (ff + 16 * FT - 1) / (16 * FT) : (ff + 64 * FT - 1) / (64 * FT);
     const long long n_wg = static_cast<long long>((max_tiles + 7) / 8 * 8) * n_groups;
     YK_REQUIRE(n_wg <= 0x7fffffffLL, "moe_gate_up: too many tiles for one launch");
     dim3 grid(static_cast<unsigned>(n_wg));
-#define YK_MOE_GU(MT, WR)                                                                                       \
-  moe_gate_up_mfma_kernel<MT, FT, WR><<<grid, 256 * WR, 0, stream>>>(                                            \
+#define YK_MOE_GU(MT, WR, KS)                                                                                   \
+  moe_gate_up_mfma_kernel<MT, FT, WR, KS><<<grid, 256 * WR, 0, stream>>>(                                            \
       static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w), order, tiles, n_tiles, top, hidden, ff, \
       kind, p0, p1, static_cast<bf16_t*>(y), n_groups)
-    if (tile_rows == 16) YK_MOE_GU(1, 1);
-    else if (tile_rows == 64) YK_MOE_GU(4, 1);
-    else YK_MOE_GU(4, 2);
+    if (tile_rows == 16) YK_MOE_GU(1, 1, true);
+    else if (tile_rows == 64) YK_MOE_GU(4, 1, false);
+    else YK_MOE_GU(4, 2, false);
 #undef YK_MOE_GU
     return yk_check_launch("moe_gate_up (matrix cores)");
   }
@@ -348,16 +395,16 @@ extern "C" int yk_moe_down(const void* y, int dtype, const void* w, int w_dtype,
   if (dtype == YK_BF16 && w_dtype == YK_BF16 && yk_moe_mfma_ok(ff, hidden, ff) && aligned16(y) && aligned16(w) &&
       aligned16(rows) && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128)) {
     constexpr int FT = 4;
-    const int n_groups = (hidden + 64 * FT - 1) / (64 * FT);
+    const int n_groups = tile_rows == 16 ? (hidden + 16 * FT - 1) / (16 * FT) : (hidden + 64 * FT - 1) / (64 * FT);
     const long long n_wg = static_cast<long long>((max_tiles + 7) / 8 * 8) * n_groups;
     YK_REQUIRE(n_wg <= 0x7fffffffLL, "moe_down: too many tiles for one launch");
     dim3 grid(static_cast<unsigned>(n_wg));
-#define YK_MOE_DN(MT, WR)                                                                                       \
-  moe_down_mfma_kernel<MT, FT, WR><<<grid, 256 * WR, 0, stream>>>(static_cast<const bf16_t*>(y), static_cast<const bf16_t*>(w), \
+#define YK_MOE_DN(MT, WR, KS)                                                                                   \
+  moe_down_mfma_kernel<MT, FT, WR, KS><<<grid, 256 * WR, 0, stream>>>(static_cast<const bf16_t*>(y), static_cast<const bf16_t*>(w), \
                                                                   order, tiles, n_tiles, hidden, ff, rows, n_groups)
-    if (tile_rows == 16) YK_MOE_DN(1, 1);
-    else if (tile_rows == 64) YK_MOE_DN(4, 1);
-    else YK_MOE_DN(4, 2);
+    if (tile_rows == 16) YK_MOE_DN(1, 1, true);
+    else if (tile_rows == 64) YK_MOE_DN(4, 1, false);
+    else YK_MOE_DN(4, 2, false);
 #undef YK_MOE_DN
     return yk_check_launch("moe_down (matrix cores)");
   }
