@@ -42,12 +42,24 @@ def dense_attention(q, k, v, positions, heads_per_kv, scale, softcap, window, ke
 @pytest.mark.parametrize("head_dim", [64, 128, 32])
 @pytest.mark.parametrize("special", [400, 399, 69, 70, 63, 64, 0, 127, 128])
 def test_one_key_stands_out_at_every_edge(dtype, head_dim, special):
+    one_key_stands_out(dtype, head_dim, special, window=200, keep=70)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window,keep,special", [(0, 0, 3), (0, 0, 321), (1000, 0, 5), (200, 0, 400), (200, 0, 401), (64, 64, 63), (64, 65, 64)])
+def test_one_far_key_among_hundreds(dtype, window, keep, special):
+    """No window at all (a far key among 700), a window larger than the sequence, a window without
+    kept first keys, and kept first keys that end at a page's border."""
+    one_key_stands_out(dtype, 64, special, window=window, keep=keep)
+
+
+def one_key_stands_out(dtype, head_dim, special, window, keep):
     """A window of 200 keys with the first 70 kept, pages of 64: one key's score towers over the
     rest; a prompt's portion at positions 550..699 and single tokens at 599, 600, 269 and 270 look
     for it.  Key 400 leaves the window between 599 and 600, keys 69 / 70 are the last kept and the
     first not kept, 63 / 64 and 127 / 128 lie across borders of pages and key blocks."""
     o = ops()
-    H, G, d, page, window, keep, L = 4, 2, head_dim, 64, 200, 70, 700
+    H, G, d, page, L = 4, 2, head_dim, 64, 700
     scale, softcap = 0.2, 30.0
     gen = torch.Generator().manual_seed(special)
     k = torch.randn(L, G, d, generator=gen) * 0.1

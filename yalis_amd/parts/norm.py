@@ -33,7 +33,8 @@ class RMSNorm(Norm):
         self.takes_embedded_rows = hasattr(rt.ops, "embedded_rows")
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.name: TensorSpec((self.size,), "float", ("one_plus_normal", 0.1))}
+        # (random weights: around the value that leaves a row as it is, 0 where 1 is added)
+        return {self.name: TensorSpec((self.size,), "float", ("normal", 0.1) if self.unit_offset else ("one_plus_normal", 0.1))}
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name]
