@@ -42,8 +42,9 @@ __device__ __forceinline__ float rotated_element(const float* buf, int i, int ro
 
 }  // namespace
 
+// A workgroup of four waves takes four heads of a token (a wave a head).
 template <typename TS, typename T, typename TW>
-__global__ __launch_bounds__(64) void qkv_prepare_kernel(
+__global__ __launch_bounds__(256) void qkv_prepare_kernel(
     const TS* __restrict__ src, int n_splits, size_t split_stride, int round_sum, int src_stride,
     T* __restrict__ q_out, int q_stride, int n_heads, int n_kv, int head_dim, int v_dim,
     const int32_t* __restrict__ positions, const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w,
@@ -51,8 +52,12 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(
     int interleaved, int max_pos, int v_norm, float v_eps, const float* __restrict__ v_cos,
     const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size, int tiled) {
-  __shared__ float buf[kMaxHead];
-  const int n = blockIdx.x, slot_y = blockIdx.y, lane = threadIdx.x;
+  __shared__ float bufs[4][kMaxHead];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  float* buf = bufs[wave];
+  const int n = blockIdx.x, n_slots = n_heads + 2 * n_kv;
+  const bool live = blockIdx.y * 4 + wave < n_slots;  // (a wave beyond the heads works on the last one and stores nothing)
+  const int slot_y = min(static_cast<int>(blockIdx.y) * 4 + wave, n_slots - 1);
   const int kind = slot_y < n_heads ? 0 : (slot_y < n_heads + n_kv ? 1 : 2);  // q, k, v
   const int len = kind == 2 ? v_dim : head_dim;
   int col0;
@@ -117,7 +122,7 @@ __global__ __launch_bounds__(64) void qkv_prepare_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int d = lane + 64 * i;
-    if (d >= len) continue;
+    if (d >= len || !live) continue;
     const float v = rot > 0 ? rotated_element(buf, d, rot, inter, cr, sr, 1.f) : buf[d];
     if (kind == 0)
       q_out[static_cast<size_t>(n) * q_stride + col0 + d] = from_f32<T>(v);
@@ -145,7 +150,7 @@ extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int 
   YK_REQUIRE(!tiled || (head_dim == v_dim && cache_is_tiled(act_dtype, head_dim, page_size)), "qkv_prepare: these pages cannot be tiled");
   YK_REQUIRE(n_heads + 2 * n_kv <= 65535, "qkv_prepare: too many heads for one launch");
   if (n_tokens == 0) return 0;
-  dim3 grid(n_tokens, n_heads + 2 * n_kv), block(64);
+  dim3 grid(n_tokens, (n_heads + 2 * n_kv + 3) / 4), block(256);
   const size_t stride = static_cast<size_t>(n_tokens) * src_stride;
 #define YK_CASE(SD, TS, AD, T, WD, TW)                                                                       \
   if (src_dtype == SD && act_dtype == AD && (norm_w_dtype == WD || (q_norm_w == nullptr && k_norm_w == nullptr && WD == YK_F32))) { \
