@@ -24,6 +24,11 @@ batch 1 / 8 / 64 behind 2,048-token prompts at the Llama-3.1-70B shape (``--no-7
 it out); ``breakdown``: the time of a
 decode step and of the prefill by kind of work (products, attention, output head, norms),
 each with the fraction of the peak that bounds it.
+
+``--design suranex`` measures instead (the default workload above is untouched): prefill and decode
+of the Suranex design at two layer sizes beside the Llama configuration of equal width, depth, heads
+and active feed-forward width, one JSON line a size, with the time of every kind of call into the
+kernel library, its bound max(bytes / 8 TB/s, flops / 2.5 PFLOP/s) and time / bound.
 """
 import argparse
 import json

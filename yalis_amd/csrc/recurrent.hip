@@ -85,9 +85,9 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
   extern __shared__ float us[];  // [kGateTokens][block_size]
   const int n0 = blockIdx.x * kGateTokens, b = blockIdx.y;
   const int count = min(kGateTokens, n_tokens - n0);
-  for (int i = threadIdx.x; i < count * block_size; i += blockDim.x) {
+  for (int i = threadIdx.x; i < kGateTokens * block_size; i += blockDim.x) {
     const int t = i / block_size, k = i % block_size;
-    us[i] = to_f32<T>(u[static_cast<size_t>(n0 + t) * channels + b * block_size + k]);
+    us[i] = t < count ? to_f32<T>(u[static_cast<size_t>(n0 + t) * channels + b * block_size + k]) : 0.f;
   }
   __syncthreads();
   const size_t mat = static_cast<size_t>(b) * block_size * block_size;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
       const float wi = to_f32<TW>(wi_t[mat + static_cast<size_t>(k) * block_size + o]);
 #pragma unroll
       for (int t = 0; t < kGateTokens; ++t) {
-        const float uv = us[t * block_size + k];  // rows beyond `count` hold stale numbers, never stored
+        const float uv = us[t * block_size + k];
         ra[t] = fmaf(wa, uv, ra[t]);
         ri[t] = fmaf(wi, uv, ri[t]);
       }
@@ -225,7 +225,17 @@ extern "C" int yk_rglru_gates(const void* u, int dtype, const void* wa_t, const 
         n_tokens, channels, block_size);
     return yk_check_launch("rglru_gates (matrix cores)");
   }
-  YK_REQUIRE(lds <= 60 * 1024, "rglru_gates: blocks of more than 960 channels do not fit the float32 form");
+  YK_REQUIRE(lds <= 150 * 1024, "rglru_gates: blocks of more than 2,400 channels do not fit the float32 form");
+  if (lds > 48 * 1024) {  // more than the default limit of dynamic LDS: raised once per kernel form
+    static bool raised = false;
+    if (!raised) {
+      bool ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&rglru_gates_kernel<float, float>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+      ok = ok && hipFuncSetAttribute(reinterpret_cast<const void*>(&rglru_gates_kernel<bf16_t, bf16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+      ok = ok && hipFuncSetAttribute(reinterpret_cast<const void*>(&rglru_gates_kernel<bf16_t, float>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+      if (!ok) return yk_fail("rglru_gates: cannot raise the LDS limit");
+      raised = true;
+    }
+  }
   dim3 grid((n_tokens + kGateTokens - 1) / kGateTokens, blocks);
   const int threads = std::min(256, (block_size + 63) / 64 * 64);
 #define YK_CASE(D, T, WD, TW)                                                                                  \

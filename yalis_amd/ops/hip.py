@@ -868,6 +868,10 @@ class HipOps:
         tiles) the caller takes a ``SplitAttention`` as well: what a step of up to 16 tokens,
         none of them in a long tile, leaves when its keys were split across workgroups.
 
+        ``keep_first`` / ``softcap`` (matrix-core kernels only; other sizes are ``attention_masked``'s): with a
+        window, the first ``keep_first`` keys of a request stay visible below it; scores times the scale
+        are squashed to softcap * tanh(s / softcap).
+
         ``rope`` (only where ``attention_can_rotate``, and only for steps whose spans are single
         tokens): ``qkv`` is then the projection's raw output (a tensor or a ``SplitSum``) and
         the launch does what ``rope_append`` would have done before it: it rotates the queries
