@@ -108,3 +108,28 @@ def one_key_stands_out(dtype, head_dim, special, window, keep):
                               keep_first=keep, softcap=softcap)
             err = (got.float().cpu().view(-1, H, d).double() - want).abs().max(dim=2).values.max(dim=1).values
             assert err.max() < tol, f"matrix cores, plan {plan}/{long_plan}: position {int(positions[int(err.argmax())])} differs by {err.max():.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,hidden,ff,experts,top", [
+    (301, 32, 8, 1, 1), (301, 64, 8, 1, 1), (7, 64, 32, 4, 2), (70, 64, 32, 3, 1), (200, 64, 96, 2, 2), (500, 128, 64, 4, 2),
+    (300, 96, 40, 2, 1), (33, 40, 24, 5, 3), (1, 128, 32, 8, 4), (640, 32, 32, 2, 2), (260, 256, 8, 1, 1), (130, 8, 8, 1, 1),
+])
+def test_experts_every_path(dtype, n, hidden, ff, experts, top):
+    """The experts' rows against plain arithmetic at sizes that take every form of the two products:
+    float32 FMA (any sizes), straight from memory into the matrix cores with tiles of 16 and of 64
+    pairs, and tiles of 128 through LDS; widths down to 8, one expert, every expert chosen."""
+    import kernel_refs as R
+
+    gen = torch.Generator().manual_seed(n + hidden)
+    x = torch.randn(n, hidden, generator=gen).to(dtype)
+    ids = torch.randint(0, 50, (n,), generator=gen, dtype=torch.int32)
+    table = torch.rand(50, experts, generator=gen).argsort(-1)[:, :top].to(torch.int32).contiguous()
+    wgu = (torch.randn(experts, 2, ff, hidden, generator=gen) / hidden ** 0.5).to(dtype)
+    wd = (torch.randn(experts, hidden, ff, generator=gen) / ff ** 0.5).to(dtype)
+    act = ("clamped_swish", 1.5, 1.702)
+    want = R.moe_experts(x, ids, table, wgu, wd, act)
+    got = ops().moe_experts(x.cuda(), ids.cuda(), table.cuda(), wgu.cuda(), wd.cuda(), act).cpu()
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    err = (got - want).abs().max(dim=1).values
+    assert err.max() <= tol * max(1.0, float(want.abs().max())), f"row {int(err.argmax())} (token {int(err.argmax()) // top}) differs by {err.max():.3e}"
