@@ -102,3 +102,22 @@ def test_random_orders_keep_the_books(seed):
         m.release(r)
     m.audit()
     assert m.free_pages(0) == n_pages and m.free_pages(1) == n_pages and m.free_slots() == n_slots
+
+
+def test_window_keeps_the_pages_of_kept_first_tokens():
+    """A window of 32 tokens with the first 20 kept, pages of 16: as the request grows, pages below the
+    window go back to the pool, except the two that hold kept tokens; a group without kept tokens
+    gives those back too."""
+    m = PageManager(16, [GroupShape(16, window=32, keep_first=20), GroupShape(16, window=32)], num_slots=1)
+    m.admit(7)
+    assert m.reserve(7, 200)
+    m.advance(7, 200)
+    kept, plain = m.block_table(7, 0).tolist(), m.block_table(7, 1).tolist()
+    # keys below 200 - 32 + 1 = 169 are dead: whole pages 0..9; the kept group holds on to pages 0 and 1
+    assert [p >= 0 for p in kept] == [True, True] + [False] * 8 + [True] * 3
+    assert [p >= 0 for p in plain] == [False] * 10 + [True] * 3
+    assert m.free_pages(0) == 16 - 5 and m.free_pages(1) == 16 - 3
+    m.audit()
+    m.release(7)
+    assert m.free_pages(0) == 16 and m.free_pages(1) == 16
+    m.audit()
