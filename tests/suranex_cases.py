@@ -76,8 +76,7 @@ def random_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
     out = {}
     for name, spec in tensor_specs_for(cfg).items():
         if spec.kind == "int":
-            experts = max(int(layer["mlp"]["router"]["experts"]) for layer in cfg["layers"] if layer["mlp"] is not None
-                          and name.startswith(f"l{cfg['layers'].index(layer)}."))
+            experts = int(cfg["layers"][int(name.split(".")[0][1:])]["mlp"]["router"]["experts"])  # "l<i>.mlp.table"
             out[name] = torch.rand((*spec.shape[:-1], experts), generator=g).argsort(-1)[..., : spec.shape[-1]].to(torch.int32)
             continue
         last = name.rsplit(".", 1)[-1]

@@ -157,9 +157,12 @@ def test_each_mechanism_alone(backend, which):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-def test_greedy_generation_through_the_engine(tmp_path, backend):
+@pytest.mark.parametrize("num_pages", [24, 7])
+def test_greedy_generation_through_the_engine(tmp_path, backend, num_pages):
     """``LLMEngine.generate`` with the scheduler under a token budget that cuts prompts into
-    portions: greedy tokens are the plain implementation's wherever its two best logits are clearly apart."""
+    portions, and with so few pages that the youngest request is preempted and starts again (its
+    state slot cleared): greedy tokens are the plain implementation's wherever its two best logits
+    are clearly apart."""
     from yalis_amd import EngineConfig, InferenceConfig, LLMEngine, ModelConfig
     from yalis_amd.weights.safetensors_io import write_dict
 
@@ -177,12 +180,14 @@ def test_greedy_generation_through_the_engine(tmp_path, backend):
         ModelConfig(model_path=str(folder), precision=precision),
         InferenceConfig(max_batch_size=3, max_length_of_generated_sequences=128, temperature=0.0),
         device=device, ops=RefOps() if device == "cpu" else None,
-        engine_config=EngineConfig(page_size=16, num_pages=24, max_num_seqs=3, max_model_len=128, max_num_batched_tokens=24,
+        engine_config=EngineConfig(page_size=16, num_pages=num_pages, max_num_seqs=3, max_model_len=128, max_num_batched_tokens=24,
                                    dtype=dtype, device=device),
     )
     prompts = list(X.make_requests(cfg, [30, 7, 45], seed=4).values())
-    out, _ = eng.generate(prompts, tokens_to_generate=12)
+    out, metrics = eng.generate(prompts, tokens_to_generate=12)
     assert out.shape == (3, 12)
+    if num_pages == 7:
+        assert metrics["Preemptions"] > 0, "this pool was meant to force a preemption"
     gap = 0.2 if dtype == "bfloat16" else 1e-3
     for prompt, row in zip(prompts, out.tolist()):
         toks = list(prompt)

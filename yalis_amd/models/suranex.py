@@ -70,7 +70,7 @@ class SuranexConfig:
             mr = KeyReader(mask, where=where + " mask")
             out["window"] = mr.integer("size", default=None, minimum=1)
             out["keep_first"] = mr.integer("keep_first", default=0, minimum=0)
-            mr.finish(strict=True)
+            mr.finish()
         rot = KeyReader(r.mapping("rot"), where=where + " rot")
         out["rot_base"] = rot.number("base", positive=True)
         out["rot_dims"] = rot.integer("dims", minimum=2)
@@ -84,9 +84,9 @@ class SuranexConfig:
                 "kind": "yarn", "factor": sr.number("factor", positive=True), "original": sr.number("original", positive=True),
                 "fast": sr.number("fast", positive=True), "slow": sr.number("slow", positive=True),
             }
-            sr.finish(strict=True)
-        rot.finish(strict=True)
-        r.finish(strict=True)
+            sr.finish()
+        rot.finish()
+        r.finish()
         return out
 
     @staticmethod
@@ -95,7 +95,7 @@ class SuranexConfig:
         out = {"width": r.integer("width", minimum=1), "blocks": r.integer("blocks", minimum=1), "conv": r.integer("conv", minimum=1)}
         if out["width"] % out["blocks"]:
             raise ConfigError(f"{where}: width={out['width']} does not divide into {out['blocks']} blocks")
-        r.finish(strict=True)
+        r.finish()
         return out
 
     @staticmethod
@@ -114,10 +114,10 @@ class SuranexConfig:
         if shared is not None:
             sr = KeyReader(shared, where=where + " shared")
             out["shared"] = {"ff": sr.integer("ff", minimum=1), "limit": sr.number("limit", positive=True)}
-            sr.finish(strict=True)
-        router.finish(strict=True)
-        expert.finish(strict=True)
-        r.finish(strict=True)
+            sr.finish()
+        router.finish()
+        expert.finish()
+        r.finish()
         return out
 
     @classmethod
@@ -145,7 +145,7 @@ class SuranexConfig:
                 raise ConfigError(f"{where}: mixer type {kind!r} is not one of this design's ('attention', 'rglru')")
             mlp = er.mapping("mlp", default=None)
             layers.append(SuranexLayer(kind, m, None if mlp is None else cls._mlp(mlp, where + " mlp")))
-            er.finish(strict=True)
+            er.finish()
         r.taken.add("architecture")
         r.finish(strict=strict)
         return cls(vocab, width, eps, tuple(layers), dict(raw))
