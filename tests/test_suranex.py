@@ -198,3 +198,43 @@ def test_greedy_generation_through_the_engine(tmp_path, backend, num_pages):
                 break  # too close to call; what follows would compare other sequences
             assert t == int(torch.argmax(logits)), f"generated {row}, the plain implementation differs after {len(toks) - len(prompt)} tokens"
             toks.append(t)
+
+
+def test_config_reader_and_spec():
+    """Sizes and constants come from config.json; what cannot run is refused with the key's name; the
+    tensors a model asks for are the design's names and shapes."""
+    import copy
+
+    from yalis_amd.config.reader import ConfigError
+    from yalis_amd.engine.factory import spec_from_config, tensor_specs_for
+
+    cfg = X.CONFIGS["mix"]
+    _, typed, spec = spec_from_config(cfg)
+    assert spec.vocab_size == 128 and spec.hidden_size == 64 and len(spec.layers) == 5
+    att = spec.layers[1].parts["mixer"].params
+    assert (att["window"], att["keep_first"], att["softcap"], att["value_dim"], att["head_dim"]) == (20, 5, 30.0, 32, 32)
+    assert att["position"].params["scaling"]["kind"] == "yarn" and att["position"].params["rotary_dim"] == 16
+    assert spec.layers[2].parts["mixer"].params["window"] is None, "no mask: every earlier key"
+    assert "feed_forward" not in spec.layers[2].parts and "feed_forward" in spec.layers[0].parts
+    assert spec.layers[4].parts["mixer"].kind == "rglru" and spec.layers[4].parts["mixer"].params["conv_taps"] == 5
+    specs = tensor_specs_for(cfg)
+    assert specs["l0.mix.ra"].shape == (1, 64, 64) and specs["l0.mix.conv"].shape == (64, 2) and specs["l0.mlp.table"].shape == (128, 3)
+    assert specs["l1.mix.g"].shape == (4, 64) and specs["l1.mix.q.norm"].shape == (32,) and specs["l2.mix.o"].shape == (64, 2 * 64)
+    assert specs["l0.mlp.shared.gate"].shape == (64, 64) and "l1.mlp.shared.gate" not in specs and "l2.norm2" not in specs
+    for path, value, what in [
+        (("layers", 1, "mixer", "kv_heads"), 3, "multiple"), (("layers", 1, "mixer", "vdim"), 7, "even"),
+        (("layers", 1, "mixer", "rot", "dims"), 40, "at most"), (("layers", 0, "type"), "conv", "not one of"),
+        (("layers", 0, "mixer", "blocks"), 5, "divide"), (("layers", 0, "mlp", "router", "top"), 9, "top"),
+        (("layers", 0, "mlp", "kind"), "dense", "not supported"),
+    ]:
+        bad = copy.deepcopy(cfg)
+        node = bad
+        for key in path[:-1]:
+            node = node[key]
+        node[path[-1]] = value
+        with pytest.raises(ConfigError, match=what):
+            spec_from_config(bad)
+    missing = copy.deepcopy(cfg)
+    del missing["layers"][1]["mixer"]["scale"]
+    with pytest.raises(ConfigError, match="scale"):
+        spec_from_config(missing)
