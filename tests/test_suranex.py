@@ -123,6 +123,12 @@ def test_long_prompt_in_one_step(backend, name):
     runner = X.make_runner(cfg, weights, dtype, device, ops_for(device), X.PAGE[name], 16, max_seqs=1)
     got, _ = C.run_trace(runner, C.trace_tail(reqs, tail=6))
     X.assert_matches(got, want, dtype == "bfloat16", f"{name}/long prompt")
+    # the same prompt in portions: the windows give pages back on the way, and later portions read
+    # kept first keys from pages that stayed beside keys whose pages are gone
+    runner = X.make_runner(cfg, weights, dtype, device, ops_for(device), X.PAGE[name], 16, max_seqs=1)
+    got, rp = C.run_trace(runner, C.trace_portions(reqs, sizes=[70, 2, 33, 64, 5, 100]))
+    X.assert_matches(got, want, dtype == "bfloat16", f"{name}/long prompt in portions")
+    assert any(p < 0 for tables in rp.page_log[-2]["r0"] for p in tables), "some window was meant to give pages back"
 
 
 def _one_layer(layer, mlp):
