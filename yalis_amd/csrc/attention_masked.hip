@@ -65,6 +65,36 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
   else if (kind == 1) col0 = n_heads * head_dim + (slot_y - n_heads) * head_dim;
   else col0 = (n_heads + n_kv) * head_dim + (slot_y - n_heads - n_kv) * v_dim;
   const TS* row = src + static_cast<size_t>(n) * src_stride + col0;
+  // the position, this lane's cosines and sines and the token's slot are asked for before the row
+  // is: three waits for memory one behind the other (position, table, row) become two side by side
+  const int pos = positions[n];
+  const float *cr = nullptr, *sr = nullptr;
+  int rot = 0, inter = 0;
+  if (kind == 2) {
+    if (v_cos != nullptr) {
+      const int p = min(pos, v_max_pos - 1);
+      rot = v_dim, inter = v_interleaved;
+      cr = v_cos + static_cast<size_t>(p) * (v_dim / 2);
+      sr = v_sin + static_cast<size_t>(p) * (v_dim / 2);
+    }
+  } else if (rotary_dim > 0) {
+    const int p = min(pos, max_pos - 1);
+    rot = rotary_dim, inter = interleaved;
+    cr = cos_t + static_cast<size_t>(p) * (rotary_dim / 2);
+    sr = sin_t + static_cast<size_t>(p) * (rotary_dim / 2);
+  }
+  float cv[4], sv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    cv[i] = 1.f, sv[i] = 0.f;
+    if (d < rot) {
+      const int m = inter ? d / 2 : (d < rot / 2 ? d : d - rot / 2);
+      cv[i] = cr[m];
+      sv[i] = sr[m];
+    }
+  }
+  const int slot = kind != 0 ? slots[n] : 0;
   float val[4];
   float ss = 0.f;
 #pragma unroll
@@ -95,26 +125,9 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
     if (d < len) buf[d] = val[i];
   }
   __syncthreads();
-  const int pos = positions[n];
-  const float *cr = nullptr, *sr = nullptr;
-  int rot = 0, inter = 0;
-  if (kind == 2) {
-    if (v_cos != nullptr) {
-      const int p = min(pos, v_max_pos - 1);
-      rot = v_dim, inter = v_interleaved;
-      cr = v_cos + static_cast<size_t>(p) * (v_dim / 2);
-      sr = v_sin + static_cast<size_t>(p) * (v_dim / 2);
-    }
-  } else if (rotary_dim > 0) {
-    const int p = min(pos, max_pos - 1);
-    rot = rotary_dim, inter = interleaved;
-    cr = cos_t + static_cast<size_t>(p) * (rotary_dim / 2);
-    sr = sin_t + static_cast<size_t>(p) * (rotary_dim / 2);
-  }
   size_t base = 0;
   int off = 0;
   if (kind != 0) {
-    const int slot = slots[n];
     const int page = slot / page_size, g = kind == 1 ? slot_y - n_heads : slot_y - n_heads - n_kv;
     off = slot % page_size;
     base = (static_cast<size_t>(page) * n_kv + g) * page_size * (kind == 1 ? head_dim : v_dim);
@@ -123,7 +136,13 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
   for (int i = 0; i < 4; ++i) {
     const int d = lane + 64 * i;
     if (d >= len || !live) continue;
-    const float v = rot > 0 ? rotated_element(buf, d, rot, inter, cr, sr, 1.f) : buf[d];
+    float v = buf[d];
+    if (d < rot) {  // the pair's other element from LDS, the angle from the registers
+      if (inter)
+        v = (d % 2 == 0) ? rot_first(buf[d], buf[d + 1], cv[i], sv[i]) : rot_second(buf[d - 1], buf[d], cv[i], sv[i]);
+      else
+        v = d < rot / 2 ? rot_first(buf[d], buf[d + rot / 2], cv[i], sv[i]) : rot_second(buf[d - rot / 2], buf[d], cv[i], sv[i]);
+    }
     if (kind == 0)
       q_out[static_cast<size_t>(n) * q_stride + col0 + d] = from_f32<T>(v);
     else if (kind == 1)
