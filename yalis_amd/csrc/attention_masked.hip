@@ -152,6 +152,153 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
   }
 }
 
+// The same for many tokens of bfloat16: a workgroup of eight waves takes one head of eight
+// consecutive tokens of the batch (a wave a token), leaves the finished heads in LDS and stores
+// them in pieces of 16 bytes: eight elements of a query or key row, and, where the eight tokens'
+// slots run on from a multiple of eight within a page, the eight tokens' values of one element as
+// one piece of the transposed page (a token at a time stores each value two bytes wide into a
+// row of its own, 128 bytes from the next).
+template <typename TS, typename TW>
+__global__ __launch_bounds__(512) void qkv_prepare8_kernel(
+    const TS* __restrict__ src, int n_splits, size_t split_stride, int round_sum, int src_stride,
+    bf16_t* __restrict__ q_out, int q_stride, int n_heads, int n_kv, int head_dim, int v_dim,
+    const int32_t* __restrict__ positions, const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w,
+    int qk_norm, float qk_eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim,
+    int interleaved, int max_pos, int v_norm, float v_eps, const float* __restrict__ v_cos,
+    const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, bf16_t* __restrict__ k_cache,
+    bf16_t* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size, int tiled, int n_tokens) {
+  __shared__ float bufs[8][kMaxHead];
+  __shared__ __attribute__((aligned(16))) bf16_t outs[8][kMaxHead];
+  __shared__ int slot_s[8];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  float* buf = bufs[wave];
+  const int n0 = blockIdx.x * 8, n_live = min(8, n_tokens - n0);
+  const int n = min(n0 + wave, n_tokens - 1);  // (a wave beyond the tokens repeats the last one; nothing of it is stored)
+  const int slot_y = blockIdx.y;
+  const int kind = slot_y < n_heads ? 0 : (slot_y < n_heads + n_kv ? 1 : 2);  // q, k, v: the same for the workgroup
+  const int len = kind == 2 ? v_dim : head_dim;
+  int col0;
+  if (kind == 0) col0 = slot_y * head_dim;
+  else if (kind == 1) col0 = n_heads * head_dim + (slot_y - n_heads) * head_dim;
+  else col0 = (n_heads + n_kv) * head_dim + (slot_y - n_heads - n_kv) * v_dim;
+  const TS* row = src + static_cast<size_t>(n) * src_stride + col0;
+  const int pos = positions[n];
+  const float *cr = nullptr, *sr = nullptr;
+  int rot = 0, inter = 0;
+  if (kind == 2) {
+    if (v_cos != nullptr) {
+      const int p = min(pos, v_max_pos - 1);
+      rot = v_dim, inter = v_interleaved;
+      cr = v_cos + static_cast<size_t>(p) * (v_dim / 2);
+      sr = v_sin + static_cast<size_t>(p) * (v_dim / 2);
+    }
+  } else if (rotary_dim > 0) {
+    const int p = min(pos, max_pos - 1);
+    rot = rotary_dim, inter = interleaved;
+    cr = cos_t + static_cast<size_t>(p) * (rotary_dim / 2);
+    sr = sin_t + static_cast<size_t>(p) * (rotary_dim / 2);
+  }
+  float cv[4], sv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    cv[i] = 1.f, sv[i] = 0.f;
+    if (d < rot) {
+      const int m = inter ? d / 2 : (d < rot / 2 ? d : d - rot / 2);
+      cv[i] = cr[m];
+      sv[i] = sr[m];
+    }
+  }
+  if (lane == 0) slot_s[wave] = kind != 0 ? slots[n] : 0;
+  float val[4];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    float v = 0.f;
+    if (d < len) {
+      for (int s = 0; s < n_splits; ++s) v += to_f32<TS>(row[s * split_stride + d]);
+      v = as_output(v, round_sum);
+    }
+    val[i] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const bool normed = kind == 2 ? v_norm != 0 : qk_norm != 0;
+  if (normed) {
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(len) + (kind == 2 ? v_eps : qk_eps));
+    const TW* w = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < len) val[i] = val[i] * inv * (w != nullptr ? to_f32<TW>(w[d]) : 1.f);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < len) buf[d] = val[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d >= len) continue;
+    float v = buf[d];
+    if (d < rot) {
+      if (inter)
+        v = (d % 2 == 0) ? rot_first(buf[d], buf[d + 1], cv[i], sv[i]) : rot_second(buf[d - 1], buf[d], cv[i], sv[i]);
+      else
+        v = d < rot / 2 ? rot_first(buf[d], buf[d + rot / 2], cv[i], sv[i]) : rot_second(buf[d - rot / 2], buf[d], cv[i], sv[i]);
+    }
+    outs[wave][d] = f32_to_bf16(v);
+  }
+  __syncthreads();
+  const int pieces = len / 8;  // (len is a multiple of 8 here)
+  if (kind == 0) {
+    for (int idx = threadIdx.x; idx < n_live * pieces; idx += blockDim.x) {
+      const int t = idx / pieces, p = idx % pieces;
+      *reinterpret_cast<uint4*>(q_out + static_cast<size_t>(n0 + t) * q_stride + col0 + 8 * p) =
+          *reinterpret_cast<const uint4*>(&outs[t][8 * p]);
+    }
+    return;
+  }
+  const int g = kind == 1 ? slot_y - n_heads : slot_y - n_heads - n_kv;
+  const size_t slab = static_cast<size_t>(page_size) * len;
+  if (kind == 1) {
+    for (int idx = threadIdx.x; idx < n_live * pieces; idx += blockDim.x) {
+      const int t = idx / pieces, p = idx % pieces;
+      const int slot = slot_s[t];
+      const size_t base = (static_cast<size_t>(slot / page_size) * n_kv + g) * slab;
+      *reinterpret_cast<uint4*>(k_cache + base + cache_k_offset(tiled, page_size, head_dim, slot % page_size, 8 * p)) =
+          *reinterpret_cast<const uint4*>(&outs[t][8 * p]);
+    }
+    return;
+  }
+  bool together = n_live == 8 && slot_s[0] % 8 == 0;
+#pragma unroll
+  for (int t = 1; t < 8; ++t) together = together && slot_s[t] == slot_s[0] + t;
+  if (together) {
+    const int slot = slot_s[0];
+    const size_t base = (static_cast<size_t>(slot / page_size) * n_kv + g) * slab;
+    for (int d = threadIdx.x; d < v_dim; d += blockDim.x) {
+      uint4 w;
+      w.x = outs[0][d] | (static_cast<uint32_t>(outs[1][d]) << 16);
+      w.y = outs[2][d] | (static_cast<uint32_t>(outs[3][d]) << 16);
+      w.z = outs[4][d] | (static_cast<uint32_t>(outs[5][d]) << 16);
+      w.w = outs[6][d] | (static_cast<uint32_t>(outs[7][d]) << 16);
+      *reinterpret_cast<uint4*>(v_cache + base + cache_v_offset(tiled, page_size, v_dim, slot % page_size, d)) = w;
+    }
+    return;
+  }
+  for (int idx = threadIdx.x; idx < n_live * v_dim; idx += blockDim.x) {
+    const int t = idx / v_dim, d = idx % v_dim;
+    const int slot = slot_s[t];
+    const size_t base = (static_cast<size_t>(slot / page_size) * n_kv + g) * slab;
+    v_cache[base + cache_v_offset(tiled, page_size, v_dim, slot % page_size, d)] = outs[t][d];
+  }
+}
+
 extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int round_sum, int src_stride, void* q_out,
                               int act_dtype, int q_stride, int n_tokens, int n_heads, int n_kv, int head_dim, int v_dim,
                               const int32_t* positions, const void* q_norm_w, const void* k_norm_w, int norm_w_dtype,
@@ -169,8 +316,28 @@ extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int 
   YK_REQUIRE(!tiled || (head_dim == v_dim && cache_is_tiled(act_dtype, head_dim, page_size)), "qkv_prepare: these pages cannot be tiled");
   YK_REQUIRE(n_heads + 2 * n_kv <= 65535, "qkv_prepare: too many heads for one launch");
   if (n_tokens == 0) return 0;
-  dim3 grid(n_tokens, (n_heads + 2 * n_kv + 3) / 4), block(256);
   const size_t stride = static_cast<size_t>(n_tokens) * src_stride;
+  auto al16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (act_dtype == YK_BF16 && n_tokens >= 16 && head_dim % 8 == 0 && v_dim % 8 == 0 && q_stride % 8 == 0 && page_size % 8 == 0 &&
+      al16(q_out) && al16(k_cache) && al16(v_cache) && (norm_w_dtype == YK_BF16 || norm_w_dtype == YK_F32)) {
+    dim3 grid8((n_tokens + 7) / 8, n_heads + 2 * n_kv);
+#define YK_CASE8(SD, TS, WD, TW)                                                                              \
+  if (src_dtype == SD && (norm_w_dtype == WD || (q_norm_w == nullptr && k_norm_w == nullptr && WD == YK_F32))) { \
+    qkv_prepare8_kernel<TS, TW><<<grid8, 512, 0, stream>>>(                                                    \
+        static_cast<const TS*>(src), n_splits, stride, round_sum, src_stride, static_cast<bf16_t*>(q_out), q_stride, \
+        n_heads, n_kv, head_dim, v_dim, positions, static_cast<const TW*>(q_norm_w),                           \
+        static_cast<const TW*>(k_norm_w), qk_norm, qk_eps, cos_t, sin_t, rotary_dim, interleaved, max_pos,      \
+        v_norm, v_eps, v_cos, v_sin, v_interleaved, v_max_pos, static_cast<bf16_t*>(k_cache),                  \
+        static_cast<bf16_t*>(v_cache), slots, page_size, tiled, n_tokens);                                     \
+    return yk_check_launch("qkv_prepare (8 tokens)");                                                          \
+  }
+    YK_CASE8(YK_F32, float, YK_F32, float)
+    YK_CASE8(YK_F32, float, YK_BF16, bf16_t)
+    YK_CASE8(YK_BF16, bf16_t, YK_F32, float)
+    YK_CASE8(YK_BF16, bf16_t, YK_BF16, bf16_t)
+#undef YK_CASE8
+  }
+  dim3 grid(n_tokens, (n_heads + 2 * n_kv + 3) / 4), block(256);
 #define YK_CASE(SD, TS, AD, T, WD, TW)                                                                       \
   if (src_dtype == SD && act_dtype == AD && (norm_w_dtype == WD || (q_norm_w == nullptr && k_norm_w == nullptr && WD == YK_F32))) { \
     qkv_prepare_kernel<TS, T, TW><<<grid, block, 0, stream>>>(                                                \
