@@ -133,3 +133,57 @@ def test_experts_every_path(dtype, n, hidden, ff, experts, top):
     tol = 1e-5 if dtype == torch.float32 else 2e-2
     err = (got - want).abs().max(dim=1).values
     assert err.max() <= tol * max(1.0, float(want.abs().max())), f"row {int(err.argmax())} (token {int(err.argmax()) // top}) differs by {err.max():.3e}"
+
+
+@pytest.mark.parametrize("head_dim,value_dim,page", [(64, 64, 64), (128, 128, 32), (32, 48, 16), (64, 64, 16)])
+def test_qkv_prepare_forms_agree(head_dim, value_dim, page):
+    """The form for many tokens (a head of eight tokens per workgroup, 16-byte stores) against the form
+    for few (the same tokens in calls of 12) bit for bit, and both against plain arithmetic: norms,
+    rotations and where everything lands in plain and tiled pages, for spans that start in the
+    middle of a group of eight slots and for tokens of several requests."""
+    import kernel_refs as R
+    from yalis_amd.parts.base import Rotation
+
+    o = ops()
+    H, G, n = 4, 2, 60
+    gen = torch.Generator().manual_seed(head_dim + page)
+    cols = H * head_dim + G * (head_dim + value_dim) + 8
+    qkv = torch.randn(n, cols, generator=gen).to(torch.bfloat16)
+    # three requests: positions 3.., 0.. and 21..; their slots in pages of their own
+    positions = torch.tensor(list(range(3, 28)) + list(range(0, 10)) + list(range(21, 46)), dtype=torch.int32)
+    first_page = [0, 4, 6]
+    owner = [0] * 25 + [1] * 10 + [2] * 25
+    slots = torch.tensor([(first_page[r] + int(p) // page) * page + int(p) % page for r, p in zip(owner, positions)], dtype=torch.int32)
+    n_pages = 6 + 46 // page + 2
+    qn, kn = (1 + 0.3 * torch.randn(head_dim, generator=gen)).to(torch.bfloat16), (1 + 0.3 * torch.randn(head_dim, generator=gen)).to(torch.bfloat16)
+    ang = torch.arange(64, dtype=torch.float32)[:, None] * (100.0 ** (-torch.arange(head_dim // 4, dtype=torch.float32) / (head_dim // 4)))
+    rot = Rotation(torch.cos(ang).cuda(), torch.sin(ang).cuda(), head_dim // 2, False)
+    vang = torch.arange(64, dtype=torch.float32)[:, None] * (100.0 ** (-torch.arange(value_dim // 2, dtype=torch.float32) / (value_dim // 2)))
+    vrot = Rotation(torch.cos(vang).cuda(), torch.sin(vang).cuda(), value_dim, False)
+
+    def run(chunks):
+        k = torch.zeros(n_pages, G, page, head_dim, dtype=torch.bfloat16, device="cuda")
+        v = torch.zeros(n_pages, G, value_dim, page, dtype=torch.bfloat16, device="cuda")
+        qs = []
+        for a, b in chunks:
+            qs.append(o.qkv_prepare(qkv[a:b].cuda(), H, G, head_dim, value_dim, positions[a:b].cuda(), torch.bfloat16, q_norm=qn.cuda(),
+                                    k_norm=kn.cuda(), qk_eps=1e-6, rotation=rot, value_norm_eps=1e-6, value_rotation=vrot,
+                                    k_cache=k, v_cache=v, slots=slots[a:b].cuda(), page_size=page))
+        return torch.cat(qs).cpu(), k.cpu(), v.cpu()
+
+    many = run([(0, n)])
+    few = run([(a, min(a + 12, n)) for a in range(0, n, 12)])
+    for a, b, what in zip(many, few, ("queries", "key pages", "value pages")):
+        assert torch.equal(a, b), f"{what} differ between the two forms"
+    k_ref = torch.zeros(n_pages, G, page, head_dim, dtype=torch.bfloat16)
+    v_ref = torch.zeros(n_pages, G, value_dim, page, dtype=torch.bfloat16)
+    cpu = lambda r: Rotation(r.cos.cpu(), r.sin.cpu(), r.rotary_dim, r.interleaved)
+    q_ref = R.qkv_prepare(qkv, H, G, head_dim, value_dim, positions, torch.bfloat16, q_norm=qn, k_norm=kn, qk_eps=1e-6, rotation=cpu(rot),
+                          value_norm_eps=1e-6, value_rotation=cpu(vrot), k_cache=k_ref, v_cache=v_ref, slots=slots, page_size=page)
+    k_got, v_got = many[1], many[2]
+    if o.masked_pages_tiled(torch.bfloat16, head_dim, value_dim, page):
+        from kernel_refs import untile_cache
+
+        k_got, v_got = untile_cache(k_got, v_got)
+    assert (many[0].float() - q_ref.float()).abs().max() <= 0.04
+    assert (k_got.float() - k_ref.float()).abs().max() <= 0.04 and (v_got.float() - v_ref.float()).abs().max() <= 0.04
