@@ -60,9 +60,9 @@ CONFIGS = {
     ]),
     # the sizes the matrix-core kernels take: heads of 64 with tiled bfloat16 pages of 64 tokens, widths of 32s
     "wide": model(200, 128, 1e-6, [
-        (attention(4, 1, 64, 64, 70, 4, 64, 5000.0, 0.125, softcap=40.0, scaling=YARN_A), moe(4, 2, 64, 1.5, shared=(32, 2.0))),
-        (rglru(128, 4, 4), moe(4, 2, 96, 1.5)),
-        (attention(2, 2, 128, 128, 33, 17, 32, 5000.0, 0.09, softcap=20.0), moe(8, 4, 32, 3.0, shared=(96, 1.0))),
+        (attention(4, 1, 64, 64, 70, 4, 64, 5000.0, 0.11, softcap=40.0, scaling=YARN_A), moe(4, 2, 64, 1.25, shared=(32, 2.5))),
+        (rglru(128, 2, 3), moe(4, 2, 96, 1.25)),
+        (attention(2, 2, 128, 128, 33, 17, 32, 5000.0, 0.09, softcap=20.0), moe(8, 4, 32, 3.0, shared=(64, 1.0))),
     ]),
 }
 PAGE = {"odd": 16, "mix": 32, "wide": 64}

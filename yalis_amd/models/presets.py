@@ -51,9 +51,9 @@ def suranex_shape(width: int, vocab: int, heads: int, kv_heads: int, dim: int, w
                   experts: int, top: int, ff: int, shared_ff: int, pattern=("attention", "attention", "rglru"), repeats: int = 2) -> dict:
     """A Suranex config.json of the given layer sizes: ``pattern`` repeated ``repeats`` times, every
     layer with a mixture of experts and a shared expert."""
-    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 50.0,
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 30.0,
            "mask": {"size": window, "keep_first": 4},
-           "rot": {"base": 10000.0, "dims": dim, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+           "rot": {"base": 10000.0, "dims": dim, "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
     rec = {"width": recurrent_width, "blocks": blocks, "conv": 4}
     mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff, "limit": 7.0},
            "shared": {"ff": shared_ff, "limit": 7.0}}
