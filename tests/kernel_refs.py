@@ -431,3 +431,163 @@ RefOps.attention_finish = staticmethod(attention_finish)
 RefOps.causal_conv = staticmethod(causal_conv)
 RefOps.rglru = staticmethod(rglru)
 RefOps.moe_experts = staticmethod(moe_experts)
+
+
+# ------------------------------------------------- norms on both sides of a branch, plain feed-forward
+def _norm_rows(x, constants):
+    weight, bias, eps, center = constants
+    if center:
+        x = x - x.mean(dim=-1, keepdim=True)
+    y = x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps) * weight.to(torch.float32)
+    return y if bias is None else y + bias.to(torch.float32)
+
+
+def sandwich_norm(residual, branch, post, scale, pre, rows, out_dtype):
+    """residual (float32, in place unless ``rows`` picks some) += scale * post(branch); returns
+    pre(residual) in ``out_dtype`` (None without ``pre``).  Without a residual: pre(branch)."""
+    b = None if branch is None else branch.float()
+    if residual is None:
+        return _norm_rows(b, pre).to(out_dtype)
+    if rows is not None:
+        idx = rows.long()
+        r = residual[idx]
+        if b is not None:
+            r = r + scale * (_norm_rows(b[idx], post) if post is not None else b[idx])
+    else:
+        if b is not None:
+            residual += scale * (_norm_rows(b, post) if post is not None else b)
+        r = residual
+    return None if pre is None else _norm_rows(r, pre).to(out_dtype)
+
+
+def activation(x, kind, out_dtype):
+    x = x.float()
+    if kind == "relu2":
+        y = torch.relu(x) ** 2
+    elif kind == "silu":
+        y = x * torch.sigmoid(x)
+    else:
+        y = 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x**3)))
+    return y.to(out_dtype)
+
+
+def scale_rows(x, s):
+    x *= s
+    return x
+
+
+# ------------------------------------------------------------- attention over one latent per token
+def latent_prepare(proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, rot_dim=0, kv_norm=None, rotation=None,
+                   positions=None, pages=None, slots=None, page_size=0):
+    p = proj.float()
+    c_q = _rmsnorm(p[:, :q_rank], q_norm, eps, False).to(act_dtype)
+    if kv_rank:
+        c = _rmsnorm(p[:, kv_col: kv_col + kv_rank], kv_norm, eps, False)
+        pos = positions.long()
+        r = _turn(p[:, kv_col + kv_rank: kv_col + kv_rank + rot_dim], rotation.cos[pos], rotation.sin[pos], rot_dim, rotation.interleaved)
+        row = torch.cat([c, r], dim=1).to(pages.dtype)
+        s = slots.long()
+        pages[s // page_size, 0, s % page_size, :] = row
+    return c_q
+
+
+def head_linear(x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0):
+    """Per head, out[n, h, :out_dim] = x[n, h, :in_dim] . w[h] (w [heads, in, out]); ``tail`` more elements of
+    every head of x follow the product, turned by the token's position; ``gate``: the head's output times
+    the sigmoid of column gate_col + h of ``gate``."""
+    n = x.shape[0]
+    xh = x.float().reshape(n, n_heads, in_dim + tail)
+    out = torch.einsum("nhi,hio->nho", xh[..., :in_dim], w.float())
+    if tail:
+        pos = positions.long()
+        t = _turn(xh[..., in_dim:], rotation.cos[pos][:, None, :], rotation.sin[pos][:, None, :], tail, rotation.interleaved)
+        out = torch.cat([out, t], dim=-1)
+    if gate is not None:
+        out = out * torch.sigmoid(gate[:, gate_col: gate_col + n_heads].float())[:, :, None]
+    return out.reshape(n, -1).to(out_dtype)
+
+
+def latent_attention(q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None):
+    a = ctx.arrays
+    n = q_lat.shape[0]
+    width = kv_rank + rot_dim
+    q = q_lat.float().view(n, n_heads, width)
+    out = torch.zeros((n, n_heads, kv_rank), dtype=torch.float32, device=q_lat.device)
+    bt = a[f"block_table_g{group}"]
+    for t in range(n):
+        seq, p = int(a["token_seq"][t]), int(a["positions"][t])
+        idx = torch.arange(p + 1)
+        rows = pages[bt[seq, idx // page_size].long(), 0, idx % page_size, :].float()
+        prob = torch.softmax((q[t] @ rows.T) * scale, dim=-1)
+        out[t] = prob @ rows[:, :kv_rank]
+    return out.view(n, n_heads * kv_rank)
+
+
+# ---------------------------------------------------------------- a matrix per head as the memory
+def causal_conv_act(x, weight, bias, state, ctx, act=None):
+    y = causal_conv(x, weight, bias, state, ctx)
+    return y if act is None else activation(y, act, y.dtype)
+
+
+def conv_state_push(x, state, ctx):
+    a = ctx.arrays
+    keep = state.shape[1]
+    for s in range(a["seq_qstart"].numel()):
+        q0, ql, slot = int(a["seq_qstart"][s]), int(a["seq_qlen"][s]), int(a["state_slots"][s])
+        state[slot] = torch.cat([state[slot], x[q0: q0 + ql].to(state.dtype)], dim=0)[-keep:]
+
+
+def linear_state_scan(qkv, n_heads, n_kv, dim, vdim, state, ctx, q_scale=1.0, unit_eps=None, decay=None, beta=None):
+    a = ctx.arrays
+    n = qkv.shape[0]
+    x = qkv.float()
+    kd = n_kv * dim
+    q, k, v = x[:, :kd].reshape(n, n_kv, dim), x[:, kd: 2 * kd].reshape(n, n_kv, dim), x[:, 2 * kd: 2 * kd + n_heads * vdim].reshape(n, n_heads, vdim)
+    if unit_eps is not None:
+        q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps)
+        k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)
+    q = q * q_scale
+    if decay[0] == "head":
+        _, src, col, a_log, dt_bias = decay
+        g = torch.exp(-torch.exp(a_log.float()) * torch.nn.functional.softplus(src[:, col: col + n_heads].float() + dt_bias.float()))
+        g = g[:, :, None].expand(n, n_heads, dim)
+    else:
+        _, src, col, bias, tau = decay
+        z = src[:, col: col + n_heads * dim].float() + bias.float()
+        g = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(n, n_heads, dim)
+    b = None if beta is None else torch.sigmoid(beta[0][:, beta[1]: beta[1] + n_heads].float())
+    out = torch.empty((n, n_heads, vdim), dtype=torch.float32, device=qkv.device)
+    per = n_heads // n_kv
+    for s in range(a["seq_qstart"].numel()):
+        q0, ql, slot = int(a["seq_qstart"][s]), int(a["seq_qlen"][s]), int(a["state_slots"][s])
+        S = state[slot].clone()
+        for t in range(q0, q0 + ql):
+            for h in range(n_heads):
+                kk, qq = k[t, h // per], q[t, h // per]
+                Sh = g[t, h][:, None] * S[h]
+                u = v[t, h] if b is None else b[t, h] * (v[t, h] - Sh.T @ kk)
+                Sh = Sh + torch.outer(kk, u)
+                out[t, h] = Sh.T @ qq
+                S[h] = Sh
+        state[slot] = S
+    return out.view(n, n_heads * vdim)
+
+
+def gated_head_norm(o, weight, eps, gate, gate_col, n_heads, vdim, out_dtype):
+    n = o.shape[0]
+    y = _rmsnorm(o.float().view(n, n_heads, vdim), weight, eps, False).reshape(n, -1)
+    g = gate[:, gate_col: gate_col + n_heads * vdim].float()
+    return (y * g * torch.sigmoid(g)).to(out_dtype)
+
+
+RefOps.sandwich_norm = staticmethod(sandwich_norm)
+RefOps.activation = staticmethod(activation)
+RefOps.scale_rows = staticmethod(scale_rows)
+RefOps.latent_prepare = staticmethod(latent_prepare)
+RefOps.head_linear = staticmethod(head_linear)
+RefOps.latent_attention = staticmethod(latent_attention)
+RefOps.latent_tile_tokens = staticmethod(lambda n_heads: 16 // min(n_heads, 4))
+RefOps.causal_conv = staticmethod(causal_conv_act)
+RefOps.conv_state_push = staticmethod(conv_state_push)
+RefOps.linear_state_scan = staticmethod(linear_state_scan)
+RefOps.gated_head_norm = staticmethod(gated_head_norm)

@@ -39,6 +39,14 @@ class LayerSpec:
     prefix: str
     block: str  # block-arrangement registry key, e.g. "prenorm"
     parts: Mapping[str, PartSpec] = field(default_factory=dict)  # role -> part
+    # constants of the arrangement itself (a multiplier on its branches, say), handed to it as
+    # keyword arguments beside its parts
+    params: Mapping[str, Any] = field(default_factory=dict)
+
+    def with_params(self, **params: Any) -> "LayerSpec":
+        merged = dict(self.params)
+        merged.update(params)
+        return LayerSpec(self.prefix, self.block, self.parts, merged)
 
     @classmethod
     def of(cls, prefix: str, block: str, **parts: Optional[PartSpec]) -> "LayerSpec":

@@ -1,0 +1,378 @@
+// Attention over one latent row per token.  A page row holds [c (kv_rank) | kr (rot_dim)]: the
+// normed latent from which every head's keys and values are made, and one rotated key part
+// shared by the heads.  The up-projections are applied to the queries and to the attention's
+// result instead of to the cached rows:
+//   score_h(i, j) = ([W_uk,h^T q_h,i | turn(qr_h,i)] . [c_j | kr_j]) * scale        (float32)
+//   o_h,i         = W_uv,h (sum_j softmax_j(score_h(i, .)) c_j)
+// so the pages are read as they are, all heads against the same rows.
+//
+// Three kernels:
+//   * latent_prepare: from the stacked down-projection's rows, the normed query latent, and the
+//     token's page row (normed latent, rotated key part);
+//   * head_linear: per head x[n, h, :in] . W[h] (W [heads][in][out]), with optionally a tail of
+//     every head copied behind the product turned by the token's position (queries into the
+//     latent's space) or a sigmoid gate per head on the output (values out of it);
+//   * latent_attention: a workgroup takes a tile of consecutive tokens of a request and a group
+//     of heads (16 pairs at most, four to a wave), walks the keys in blocks staged once in LDS,
+//     a lane to a key for the scores and a lane to a latent column for the weighted sum.
+#include <algorithm>
+
+#include "common.h"
+
+// --------------------------------------------------------------------------------- prepare
+template <typename T, typename TW>
+__global__ __launch_bounds__(128) void latent_prepare_kernel(
+    const T* __restrict__ proj, int proj_stride, int q_rank, const TW* __restrict__ q_norm, float eps, T* __restrict__ c_q,
+    int kv_col, int kv_rank, int rot_dim, const TW* __restrict__ kv_norm, const int32_t* __restrict__ positions,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int interleaved, T* __restrict__ pages,
+    const int32_t* __restrict__ slots) {
+  __shared__ float scratch[17];
+  const size_t n = blockIdx.x;
+  const T* row = proj + n * proj_stride;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < q_rank; c += blockDim.x) {
+    const float v = to_f32<T>(row[c]);
+    ss = fmaf(v, v, ss);
+  }
+  float inv = 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(q_rank) + eps);
+  for (int c = threadIdx.x; c < q_rank; c += blockDim.x)
+    c_q[n * q_rank + c] = from_f32<T>(to_f32<T>(row[c]) * inv * to_f32<TW>(q_norm[c]));
+  if (kv_rank == 0) return;
+  const T* kv = row + kv_col;
+  ss = 0.f;
+  for (int c = threadIdx.x; c < kv_rank; c += blockDim.x) {
+    const float v = to_f32<T>(kv[c]);
+    ss = fmaf(v, v, ss);
+  }
+  inv = 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(kv_rank) + eps);
+  T* dst = pages + static_cast<size_t>(slots[n]) * (kv_rank + rot_dim);
+  for (int c = threadIdx.x; c < kv_rank; c += blockDim.x)
+    dst[c] = from_f32<T>(to_f32<T>(kv[c]) * inv * to_f32<TW>(kv_norm[c]));
+  const int half = rot_dim / 2;
+  const size_t p = static_cast<size_t>(positions[n]);
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+    const float a = to_f32<T>(kv[kv_rank + ia]), b = to_f32<T>(kv[kv_rank + ib]);
+    const float c = cos_t[p * half + i], s = sin_t[p * half + i];
+    dst[kv_rank + ia] = from_f32<T>(rot_first(a, b, c, s));
+    dst[kv_rank + ib] = from_f32<T>(rot_second(a, b, c, s));
+  }
+}
+
+extern "C" int yk_latent_prepare(const void* proj, int proj_stride, int dtype, int q_rank, const void* q_norm, int w_dtype,
+                                 float eps, void* c_q, int kv_col, int kv_rank, int rot_dim, const void* kv_norm,
+                                 const int32_t* positions, const float* cos_t, const float* sin_t, int interleaved,
+                                 int max_positions, void* pages, const int32_t* slots, int n_tokens, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && q_rank > 0 && kv_rank >= 0 && rot_dim >= 0 && rot_dim % 2 == 0, "latent_prepare: bad sizes");
+  YK_REQUIRE(proj_stride >= q_rank && (kv_rank == 0 || proj_stride >= kv_col + kv_rank + rot_dim),
+             "latent_prepare: the projection's rows are shorter than its sections");
+  YK_REQUIRE(kv_rank == 0 || (kv_norm != nullptr && pages != nullptr && slots != nullptr && positions != nullptr),
+             "latent_prepare: a layer that keeps a cache needs its norm, pages, slots and positions");
+  YK_REQUIRE(kv_rank == 0 || rot_dim == 0 || (cos_t != nullptr && sin_t != nullptr && max_positions > 0),
+             "latent_prepare: the rotated part needs its tables");
+  if (n_tokens == 0) return 0;
+#define YK_CASE(D, T, WD, TW)                                                                                         \
+  if (dtype == D && w_dtype == WD) {                                                                                  \
+    latent_prepare_kernel<T, TW><<<n_tokens, 128, 0, stream>>>(                                                       \
+        static_cast<const T*>(proj), proj_stride, q_rank, static_cast<const TW*>(q_norm), eps, static_cast<T*>(c_q),  \
+        kv_col, kv_rank, rot_dim, static_cast<const TW*>(kv_norm), positions, cos_t, sin_t, interleaved,              \
+        static_cast<T*>(pages), slots);                                                                               \
+    return yk_check_launch("latent_prepare");                                                                         \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
+#undef YK_CASE
+  return yk_fail("latent_prepare: unsupported dtype combination");
+}
+
+// ------------------------------------------------------------------------- per-head products
+constexpr int kHeadTokens = 8;  // tokens a workgroup multiplies by one head's matrix
+
+template <typename TX, typename TW, typename TO>
+__global__ __launch_bounds__(256) void head_linear_kernel(
+    const TX* __restrict__ x, int x_stride, const TW* __restrict__ w, TO* __restrict__ out, int out_stride, int in_dim,
+    int out_dim, int tail, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int interleaved, const TX* __restrict__ gate, int gate_stride, int gate_col,
+    int n_tokens) {
+  extern __shared__ float xs[];  // [kHeadTokens][in_dim + tail]
+  const int n0 = blockIdx.x * kHeadTokens, h = blockIdx.y;
+  const int count = min(kHeadTokens, n_tokens - n0);
+  const int xw = in_dim + tail;
+  for (int i = threadIdx.x; i < kHeadTokens * xw; i += blockDim.x) {
+    const int t = i / xw, c = i % xw;
+    xs[i] = t < count ? to_f32<TX>(x[static_cast<size_t>(n0 + t) * x_stride + h * xw + c]) : 0.f;
+  }
+  __syncthreads();
+  const TW* wh = w + static_cast<size_t>(h) * in_dim * out_dim;
+  const int ow = out_dim + tail;
+  for (int o = threadIdx.x; o < out_dim; o += blockDim.x) {
+    float acc[kHeadTokens];
+#pragma unroll
+    for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
+    for (int i = 0; i < in_dim; ++i) {
+      const float wv = to_f32<TW>(wh[static_cast<size_t>(i) * out_dim + o]);
+#pragma unroll
+      for (int t = 0; t < kHeadTokens; ++t) acc[t] = fmaf(xs[t * xw + i], wv, acc[t]);
+    }
+    for (int t = 0; t < count; ++t) {
+      float v = acc[t];
+      if (gate != nullptr) v *= 1.f / (1.f + expf(-to_f32<TX>(gate[static_cast<size_t>(n0 + t) * gate_stride + gate_col + h])));
+      out[static_cast<size_t>(n0 + t) * out_stride + h * ow + o] = from_f32<TO>(v);
+    }
+  }
+  const int half = tail / 2;
+  for (int i = threadIdx.x; i < count * half; i += blockDim.x) {
+    const int t = i / half, j = i % half;
+    const int ia = interleaved ? 2 * j : j, ib = interleaved ? 2 * j + 1 : j + half;
+    const float a = xs[t * xw + in_dim + ia], b = xs[t * xw + in_dim + ib];
+    const size_t p = static_cast<size_t>(positions[n0 + t]);
+    const float c = cos_t[p * half + j], s = sin_t[p * half + j];
+    TO* dst = out + static_cast<size_t>(n0 + t) * out_stride + h * ow + out_dim;
+    dst[ia] = from_f32<TO>(rot_first(a, b, c, s));
+    dst[ib] = from_f32<TO>(rot_second(a, b, c, s));
+  }
+}
+
+extern "C" int yk_head_linear(const void* x, int x_stride, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,
+                              int n_heads, int in_dim, int out_dim, int tail, const int32_t* positions, const float* cos_t,
+                              const float* sin_t, int interleaved, const void* gate, int gate_stride, int gate_col,
+                              int n_tokens, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && in_dim > 0 && out_dim > 0 && tail >= 0 && tail % 2 == 0, "head_linear: bad sizes");
+  YK_REQUIRE(x_stride >= n_heads * (in_dim + tail), "head_linear: the input's rows are shorter than its heads");
+  YK_REQUIRE(tail == 0 || (positions != nullptr && cos_t != nullptr && sin_t != nullptr), "head_linear: a turned tail needs positions and tables");
+  const size_t lds = static_cast<size_t>(kHeadTokens) * (in_dim + tail) * sizeof(float);
+  YK_REQUIRE(lds <= 64 * 1024, "head_linear: heads of more than 2,048 input elements do not fit");
+  if (n_tokens == 0) return 0;
+  dim3 grid((n_tokens + kHeadTokens - 1) / kHeadTokens, n_heads);
+  const int block = out_dim <= 64 ? 64 : out_dim <= 128 ? 128 : 256;
+  const int out_stride = n_heads * (out_dim + tail);
+#define YK_CASE(XD, TX, WD, TW, OD, TO)                                                                              \
+  if (x_dtype == XD && w_dtype == WD && out_dtype == OD) {                                                           \
+    head_linear_kernel<TX, TW, TO><<<grid, block, lds, stream>>>(                                                    \
+        static_cast<const TX*>(x), x_stride, static_cast<const TW*>(w), static_cast<TO*>(out), out_stride, in_dim,   \
+        out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TX*>(gate), gate_stride, gate_col,    \
+        n_tokens);                                                                                                   \
+    return yk_check_launch("head_linear");                                                                           \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float, YK_F32, float)
+#undef YK_CASE
+  return yk_fail("head_linear: unsupported dtype combination");
+}
+
+// float32 rows in (the attention's sums over the latent), the activation dtype out, the gate in the
+// activation dtype: the same arithmetic with the gate's own element type
+template <typename TW, typename TG, typename TO>
+__global__ __launch_bounds__(256) void head_linear_out_kernel(
+    const float* __restrict__ x, int x_stride, const TW* __restrict__ w, TO* __restrict__ out, int out_stride, int in_dim,
+    int out_dim, const TG* __restrict__ gate, int gate_stride, int gate_col, int n_tokens) {
+  extern __shared__ float xs[];  // [kHeadTokens][in_dim]
+  const int n0 = blockIdx.x * kHeadTokens, h = blockIdx.y;
+  const int count = min(kHeadTokens, n_tokens - n0);
+  for (int i = threadIdx.x; i < kHeadTokens * in_dim; i += blockDim.x) {
+    const int t = i / in_dim, c = i % in_dim;
+    xs[i] = t < count ? x[static_cast<size_t>(n0 + t) * x_stride + h * in_dim + c] : 0.f;
+  }
+  __syncthreads();
+  const TW* wh = w + static_cast<size_t>(h) * in_dim * out_dim;
+  for (int o = threadIdx.x; o < out_dim; o += blockDim.x) {
+    float acc[kHeadTokens];
+#pragma unroll
+    for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
+    for (int i = 0; i < in_dim; ++i) {
+      const float wv = to_f32<TW>(wh[static_cast<size_t>(i) * out_dim + o]);
+#pragma unroll
+      for (int t = 0; t < kHeadTokens; ++t) acc[t] = fmaf(xs[t * in_dim + i], wv, acc[t]);
+    }
+    for (int t = 0; t < count; ++t) {
+      float v = acc[t];
+      if (gate != nullptr) v *= 1.f / (1.f + expf(-to_f32<TG>(gate[static_cast<size_t>(n0 + t) * gate_stride + gate_col + h])));
+      out[static_cast<size_t>(n0 + t) * out_stride + h * out_dim + o] = from_f32<TO>(v);
+    }
+  }
+}
+
+extern "C" int yk_head_linear_out(const float* x, int x_stride, const void* w, int w_dtype, void* out, int out_dtype,
+                                  int n_heads, int in_dim, int out_dim, const void* gate, int gate_stride, int gate_col,
+                                  int n_tokens, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && in_dim > 0 && out_dim > 0, "head_linear_out: bad sizes");
+  YK_REQUIRE(x_stride >= n_heads * in_dim, "head_linear_out: the input's rows are shorter than its heads");
+  const size_t lds = static_cast<size_t>(kHeadTokens) * in_dim * sizeof(float);
+  YK_REQUIRE(lds <= 64 * 1024, "head_linear_out: heads of more than 2,048 input elements do not fit");
+  if (n_tokens == 0) return 0;
+  dim3 grid((n_tokens + kHeadTokens - 1) / kHeadTokens, n_heads);
+  const int block = out_dim <= 64 ? 64 : out_dim <= 128 ? 128 : 256;
+#define YK_CASE(WD, TW, OD, TO)                                                                                          \
+  if (w_dtype == WD && out_dtype == OD) {                                                                                \
+    head_linear_out_kernel<TW, TO, TO><<<grid, block, lds, stream>>>(x, x_stride, static_cast<const TW*>(w),             \
+                                                                     static_cast<TO*>(out), n_heads * out_dim, in_dim,   \
+                                                                     out_dim, static_cast<const TO*>(gate), gate_stride, \
+                                                                     gate_col, n_tokens);                                \
+    return yk_check_launch("head_linear_out");                                                                           \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t)
+#undef YK_CASE
+  return yk_fail("head_linear_out: unsupported dtype combination");
+}
+
+// --------------------------------------------------------------------------------- attention
+constexpr int kLatWaves = 4;       // waves of a workgroup
+constexpr int kLatItems = 4;       // (token, head) pairs a wave carries
+constexpr int kLatPairs = kLatWaves * kLatItems;
+
+// tiles: rows of (request, first token index in the batch, token count, first position).  Workgroup
+// (tile, head group): pair i of it is token i / heads_per_group of the tile and head
+// group * heads_per_group + i % heads_per_group; wave w carries the pairs w, w + 4, w + 8, w + 12.
+// KB keys are staged per block ([KB][width] in T, rows padded by `pad` elements); RPL latent columns a lane.
+template <typename T, int RPL>
+__global__ __launch_bounds__(64 * kLatWaves) void latent_attention_kernel(
+    const float* __restrict__ q_lat, const T* __restrict__ pages, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ block_table, int table_width, int page_size, int n_heads, int heads_per_group, int kv_rank,
+    int rot_dim, float scale, int KB, int pad, float* __restrict__ out) {
+  extern __shared__ unsigned char lds_raw[];
+  const int width = kv_rank + rot_dim, row_w = width + pad;
+  T* kblock = reinterpret_cast<T*>(lds_raw);                                             // [KB][row_w]
+  float* pbuf = reinterpret_cast<float*>(lds_raw + static_cast<size_t>(KB) * row_w * sizeof(T) + 16 -
+                                         (static_cast<size_t>(KB) * row_w * sizeof(T)) % 16);  // [kLatPairs][KB]
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int32_t* tile = tiles + 4 * blockIdx.x;
+  const int seq = tile[0], tok0 = tile[1], count = tile[2], pos0 = tile[3];
+  const int group = blockIdx.y;
+  const int n_pairs = count * heads_per_group;
+  const int last_pos = pos0 + count - 1;
+
+  // this wave's pairs
+  int tok[kLatItems], head[kLatItems], pos[kLatItems];
+  bool live[kLatItems];
+  float m[kLatItems], l[kLatItems], acc[kLatItems][RPL];
+#pragma unroll
+  for (int it = 0; it < kLatItems; ++it) {
+    const int pair = wave + it * kLatWaves;
+    const int t = pair / heads_per_group;
+    head[it] = group * heads_per_group + pair % heads_per_group;
+    live[it] = pair < n_pairs && head[it] < n_heads;
+    tok[it] = tok0 + (live[it] ? t : 0);
+    if (!live[it]) head[it] = 0;
+    pos[it] = pos0 + (live[it] ? t : 0);
+    m[it] = -INFINITY;
+    l[it] = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) acc[it][r] = 0.f;
+  }
+  const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
+
+  for (int k0 = 0; k0 <= last_pos; k0 += KB) {
+    const int nk = min(KB, last_pos + 1 - k0);
+    __syncthreads();  // the block before has been read by every wave
+    for (int i = threadIdx.x; i < nk * width; i += blockDim.x) {
+      const int j = i / width, c = i % width;
+      const int key = k0 + j;
+      const size_t slot = static_cast<size_t>(bt[key / page_size]) * page_size + key % page_size;
+      kblock[j * row_w + c] = pages[slot * width + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kLatItems; ++it) {
+      if (!live[it]) continue;  // (uniform over the wave)
+      const float* q = q_lat + (static_cast<size_t>(tok[it]) * n_heads + head[it]) * width;
+      float* pw = pbuf + (wave + it * kLatWaves) * KB;
+      // scores: a lane to a key (KB may exceed 64 never: KB <= 64)
+      float s = -INFINITY;
+      if (lane < nk && k0 + lane <= pos[it]) {
+        const T* kr = kblock + lane * row_w;
+        float d = 0.f;
+        for (int c = 0; c < width; ++c) d = fmaf(q[c], to_f32<T>(kr[c]), d);
+        s = d * scale;
+      }
+      const float m_new = fmaxf(m[it], wave_max(s));
+      const float p = s == -INFINITY ? 0.f : expf(s - m_new);
+      const float corr = m[it] == -INFINITY ? 0.f : expf(m[it] - m_new);
+      l[it] = l[it] * corr + wave_sum(p);
+      m[it] = m_new;
+      if (lane < KB) pw[lane] = p;
+      // weighted sum of the latent part: a lane to the columns lane, lane + 64, ...
+      const int visible = min(nk, pos[it] - k0 + 1);
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) acc[it][r] *= corr;
+      for (int j = 0; j < visible; ++j) {
+        const float pj = pw[j];
+        const T* kr = kblock + j * row_w;
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+          const int c = lane + r * kWave;
+          if (c < kv_rank) acc[it][r] = fmaf(pj, to_f32<T>(kr[c]), acc[it][r]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < kLatItems; ++it) {
+    if (!live[it]) continue;
+    const float inv = 1.f / l[it];
+    float* o = out + (static_cast<size_t>(tok[it]) * n_heads + head[it]) * kv_rank;
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+      const int c = lane + r * kWave;
+      if (c < kv_rank) o[c] = acc[it][r] * inv;
+    }
+  }
+}
+
+extern "C" int yk_latent_tile_tokens(int n_heads) {
+  const int hpg = n_heads < kLatItems ? n_heads : kLatItems;
+  return kLatPairs / hpg;
+}
+
+extern "C" int yk_latent_attention(const float* q_lat, const void* pages, int dtype, const int32_t* tiles, int n_tiles,
+                                   const int32_t* block_table, int table_width, int page_size, int n_heads, int kv_rank,
+                                   int rot_dim, float scale, float* out, hipStream_t stream) {
+  YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && kv_rank > 0 && rot_dim >= 0 && page_size > 0 && table_width > 0,
+             "latent_attention: bad sizes");
+  YK_REQUIRE(kv_rank <= 16 * kWave, "latent_attention: latents of more than 1,024 elements are not offered");
+  if (n_tiles == 0) return 0;
+  const int hpg = n_heads < kLatItems ? n_heads : kLatItems;
+  const int groups = (n_heads + hpg - 1) / hpg;
+  const int width = kv_rank + rot_dim;
+  const size_t esz = dtype == YK_BF16 ? 2 : 4;
+  // rows a whole number of 32-bit words long and an odd number of them apart: lanes that read the
+  // same column of different keys then meet different banks
+  int pad = 0;
+  while ((static_cast<size_t>(width + pad) * esz) % 4 != 0 || ((static_cast<size_t>(width + pad) * esz) / 4) % 2 == 0) ++pad;
+  int KB = 64;
+  while (KB > 8 && static_cast<size_t>(KB) * (width + pad) * esz > 96 * 1024) KB /= 2;
+  const size_t kbytes = static_cast<size_t>(KB) * (width + pad) * esz;
+  YK_REQUIRE(kbytes <= 128 * 1024, "latent_attention: page rows too long for the key block");
+  const size_t lds = kbytes + 16 - kbytes % 16 + static_cast<size_t>(kLatPairs) * KB * sizeof(float);
+  const int rpl = (kv_rank + kWave - 1) / kWave;
+  dim3 grid(n_tiles, groups);
+#define YK_LAUNCH(T, R)                                                                                                \
+  {                                                                                                                    \
+    auto kern = latent_attention_kernel<T, R>;                                                                         \
+    if (lds > 64 * 1024 &&                                                                                             \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,          \
+                            static_cast<int>(lds)) != hipSuccess)                                                      \
+      return yk_fail("latent_attention: the key block does not fit in LDS");                                           \
+    kern<<<grid, 64 * kLatWaves, lds, stream>>>(q_lat, static_cast<const T*>(pages), tiles, block_table, table_width,  \
+                                                page_size, n_heads, hpg, kv_rank, rot_dim, scale, KB, pad, out);       \
+    return yk_check_launch("latent_attention");                                                                        \
+  }
+#define YK_RPL(T)                      \
+  if (rpl <= 1) YK_LAUNCH(T, 1)        \
+  if (rpl <= 2) YK_LAUNCH(T, 2)        \
+  if (rpl <= 4) YK_LAUNCH(T, 4)        \
+  if (rpl <= 8) YK_LAUNCH(T, 8)        \
+  YK_LAUNCH(T, 16)
+  if (dtype == YK_F32) {
+    YK_RPL(float)
+  }
+  if (dtype == YK_BF16) {
+    YK_RPL(bf16_t)
+  }
+#undef YK_RPL
+#undef YK_LAUNCH
+  return yk_fail("latent_attention: unsupported dtype");
+}

@@ -25,7 +25,7 @@ __global__ void causal_conv_kernel(const T* __restrict__ x, int x_stride, const 
                                    const TW* __restrict__ bias, const T* __restrict__ state,
                                    const int32_t* __restrict__ token_seq, const int32_t* __restrict__ seq_qstart,
                                    const int32_t* __restrict__ state_slots, T* __restrict__ out, int channels,
-                                   int taps, size_t total) {
+                                   int taps, int act, size_t total) {
   for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const int n = static_cast<int>(i / channels), c = static_cast<int>(i % channels);
@@ -42,14 +42,16 @@ __global__ void causal_conv_kernel(const T* __restrict__ x, int x_stride, const 
         v = to_f32<T>(hist[static_cast<size_t>(taps - 1 + t - back) * channels + c]);
       acc = fmaf(to_f32<TW>(w[static_cast<size_t>(c) * taps + j]), v, acc);
     }
-    out[i] = from_f32<T>(acc);
+    out[i] = from_f32<T>(act == 1 ? act_silu(acc) : acc);
   }
 }
 
+// act: 0 none, 1 silu on the convolution's output
 extern "C" int yk_causal_conv(const void* x, int x_stride, int dtype, const void* w, const void* bias, int w_dtype,
                               const void* state, const int32_t* token_seq, const int32_t* seq_qstart,
-                              const int32_t* state_slots, void* out, int n_tokens, int channels, int taps,
+                              const int32_t* state_slots, void* out, int n_tokens, int channels, int taps, int act,
                               hipStream_t stream) {
+  YK_REQUIRE(act == 0 || act == 1, "causal_conv: unknown activation");
   YK_REQUIRE(n_tokens >= 0 && channels > 0 && taps >= 1 && x_stride >= channels, "causal_conv: bad sizes");
   YK_REQUIRE(taps == 1 || state != nullptr, "causal_conv: a convolution of several taps needs its state");
   if (n_tokens == 0) return 0;
@@ -60,7 +62,7 @@ extern "C" int yk_causal_conv(const void* x, int x_stride, int dtype, const void
     causal_conv_kernel<T, TW><<<grid, 256, 0, stream>>>(static_cast<const T*>(x), x_stride, static_cast<const TW*>(w), \
                                                         static_cast<const TW*>(bias), static_cast<const T*>(state),     \
                                                         token_seq, seq_qstart, state_slots, static_cast<T*>(out),       \
-                                                        channels, taps, total);                                         \
+                                                        channels, taps, act, total);                                    \
     return yk_check_launch("causal_conv");                                                                       \
   }
   YK_CASE(YK_F32, float, YK_F32, float)

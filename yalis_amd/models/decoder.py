@@ -76,7 +76,7 @@ class DecoderModel:
                 if family == "mixer" and not owns[i]:
                     params["projects_kv"] = False
                 built[role] = FAMILIES[family].get(part.kind)(params, rt)
-            self.blocks.append(arrangement(**built))
+            self.blocks.append(arrangement(**built, **dict(ls.params)))
 
         self.cache_groups, self.state_needs, self.sites = self._plan_memory()
         # a step may be replayed from a captured graph only if every part allows it

@@ -29,7 +29,8 @@ HOST_SOURCES = ["cache_manager.cpp"]
 # benchmark's machine probes "probe".  Every library carries runtime.hip (its error slot).
 KERNEL_LIBS = {
     "kernels": ["runtime.hip", "elementwise.hip", "gemm.hip", "gemm_tile.hip", "attention.hip", "library_gemm.hip",
-                "branch.hip", "attention_masked.hip", "recurrent.hip", "moe.hip"],
+                "branch.hip", "attention_masked.hip", "recurrent.hip", "moe.hip", "sandwich_norm.hip", "latent_attention.hip",
+                "state_scan.hip"],
     "sampling": ["runtime.hip", "sampling.hip"],
     "probe": ["runtime.hip", "probe.hip"],
 }

@@ -80,7 +80,34 @@ _SIGNATURES = {
         [_vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
-    "yk_causal_conv": ([_vp, _c_int, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_causal_conv": ([_vp, _c_int, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_sandwich_norm": (
+        [_vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _c_float, _c_int, _c_float, _vp, _vp, _c_float, _c_int, _c_int, _vp, _vp,
+         _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_activation": ([_vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_size_t, _vp], _c_int),
+    "yk_scale_rows": ([_vp, _c_float, _c_size_t, _vp], _c_int),
+    "yk_latent_prepare": (
+        [_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _vp, _vp,
+         _c_int, _vp],
+        _c_int,
+    ),
+    "yk_head_linear": (
+        [_vp, _c_int, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int,
+         _c_int, _vp],
+        _c_int,
+    ),
+    "yk_head_linear_out": ([_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_latent_tile_tokens": ([_c_int], _c_int),
+    "yk_latent_attention": ([_vp, _vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp], _c_int),
+    "yk_linear_state_scan": (
+        [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_float, _c_int, _vp, _c_int,
+         _c_int, _vp, _vp, _c_float, _vp, _c_int, _c_int, _vp, _vp],
+        _c_int,
+    ),
+    "yk_gated_head_norm": ([_vp, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _vp], _c_int),
+    "yk_conv_state_push": ([_vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_rglru_gates": ([_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _vp], _c_int),
     "yk_rglru_gates_mfma_ok": ([_c_int, _c_int], _c_int),
     "yk_rglru_scan_chunked": (
@@ -163,7 +190,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 17
+_ABI = 18
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -1208,10 +1235,13 @@ class HipOps:
         return out
 
     # ------------------------------------------------ short convolution + gated linear recurrence
-    def causal_conv(self, x, weight, bias, state, ctx) -> torch.Tensor:
+    def causal_conv(self, x, weight, bias, state, ctx, act: Optional[str] = None) -> torch.Tensor:
         """Per channel, u_t = bias + sum_j weight[c, j] * x_(t - (taps - 1 - j)) over each request's
         span; inputs before the span come from ``state`` [slots, taps - 1, channels] (not changed here).
-        ``x`` [N, channels] may be a view with a row stride."""
+        ``x`` [N, channels] may be a view with a row stride.  ``act`` = "silu": applied to u (float32)
+        before it is rounded."""
+        if act not in (None, "silu"):
+            raise KernelError(f"causal_conv: activation {act!r} is not offered")
         n, channels = x.shape
         taps = weight.shape[1]
         if x.stride(1) != 1 or tuple(weight.shape) != (channels, taps) or not weight.is_contiguous():
@@ -1226,9 +1256,233 @@ class HipOps:
             self.lib.yk_causal_conv(
                 x.data_ptr(), x.stride(0), _code(x.dtype), weight.data_ptr(), _ptr(bias), _code(weight.dtype), _ptr(state),
                 a["token_seq"].data_ptr(), a["seq_qstart"].data_ptr(), a["state_slots"].data_ptr(), out.data_ptr(),
-                n, channels, taps, self._stream(),
+                n, channels, taps, int(act == "silu"), self._stream(),
             )
         )
+        return out
+
+    # ------------------------------------------------- norms on both sides of a branch, plain feed-forward
+    def sandwich_norm(self, residual, branch, post, scale, pre, rows, out_dtype):
+        """residual (float32 [N, width], in place unless ``rows`` picks some of them) += scale *
+        post(branch); returns pre(residual) in ``out_dtype``, or None without ``pre``.  ``post`` and
+        ``pre`` are (weight, bias or None, eps, centred) or None (``post`` None: the branch is added as
+        it is); ``branch`` a tensor, a ``SplitSum`` or None.  Without a residual: pre(branch)."""
+        n_splits, round_sum, src = 1, 0, branch
+        if isinstance(branch, SplitAttention):
+            branch = src = branch.merge()
+        if isinstance(branch, SplitSum):
+            branch.check_live()
+            n_splits, round_sum, src = branch.n_splits, branch.round_sum, branch.tensor
+        ref = residual if residual is not None else branch
+        if ref is None:
+            raise KernelError("sandwich_norm: neither a residual nor a branch")
+        n, width = ref.shape
+        if residual is not None and (residual.dtype != torch.float32 or not residual.is_contiguous() or residual.dim() != 2):
+            raise KernelError("the residual stream must be contiguous float32 rows")
+        if branch is not None and (tuple(branch.shape) != (n, width) or not src.is_contiguous()):
+            raise KernelError(f"branch {tuple(branch.shape)} does not match the rows {(n, width)}")
+        if post is not None and branch is None:
+            raise KernelError("sandwich_norm: a branch's norm without a branch")
+        w_dtype = None
+        for c in (post, pre):
+            if c is None:
+                continue
+            w, b = c[0], c[1]
+            if w.numel() != width or not w.is_contiguous() or (b is not None and (b.numel() != width or b.dtype != w.dtype or not b.is_contiguous())):
+                raise KernelError(f"sandwich_norm: a norm's weight or bias does not fit rows of {width}")
+            if w_dtype not in (None, w.dtype):
+                raise KernelError("sandwich_norm: the two norms' weights differ in dtype")
+            w_dtype = w.dtype
+        n_out = n
+        if rows is not None:
+            if residual is None or rows.dtype != torch.int32 or not rows.is_contiguous():
+                raise KernelError("sandwich_norm: gathered rows need a residual and an int32 index")
+            n_out = rows.numel()
+        out = torch.empty((n_out, width), dtype=out_dtype, device=ref.device) if pre is not None else None
+        pa = post if post is not None else (None, None, 0.0, False)
+        pb = pre if pre is not None else (None, None, 0.0, False)
+        self._check(self.lib.yk_sandwich_norm(
+            _ptr(residual), _ptr(src), 0 if src is None else _code(src.dtype), n_splits, round_sum, n,
+            _ptr(pa[0]), _ptr(pa[1]), float(pa[2]), int(bool(pa[3])), float(scale), _ptr(pb[0]), _ptr(pb[1]), float(pb[2]),
+            int(bool(pb[3])), 0 if w_dtype is None else _code(w_dtype), _ptr(rows), _ptr(out), _code(out_dtype), n_out, width,
+            self._stream()))
+        return out
+
+    ACTIVATION_KINDS = {"silu": 0, "gelu_tanh": 1, "relu2": 2}
+
+    def activation(self, x, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
+        """act(x) elementwise in float32, rounded once; ``x`` a tensor or a product's unreduced slices."""
+        if kind not in self.ACTIVATION_KINDS:
+            raise KernelError(f"activation {kind!r} is not offered (offered: {sorted(self.ACTIVATION_KINDS)})")
+        n_splits, round_sum, src = 1, 0, x
+        if isinstance(x, SplitSum):
+            x.check_live()
+            n_splits, round_sum, src = x.n_splits, x.round_sum, x.tensor
+        if not src.is_contiguous():
+            raise KernelError("activation: the input must be contiguous")
+        out = torch.empty(tuple(x.shape), dtype=out_dtype, device=src.device)
+        self._check(self.lib.yk_activation(src.data_ptr(), _code(src.dtype), n_splits, round_sum, self.ACTIVATION_KINDS[kind],
+                                           out.data_ptr(), _code(out_dtype), out.numel(), self._stream()))
+        return out
+
+    def scale_rows(self, x: torch.Tensor, s: float) -> torch.Tensor:
+        """x (contiguous float32) *= s, in place."""
+        if x.dtype != torch.float32 or not x.is_contiguous():
+            raise KernelError("scale_rows takes a contiguous float32 tensor")
+        self._check(self.lib.yk_scale_rows(x.data_ptr(), float(s), x.numel(), self._stream()))
+        return x
+
+    # ------------------------------------------------------------- attention over one latent per token
+    def latent_prepare(self, proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, rot_dim=0, kv_norm=None, rotation=None,
+                       positions=None, pages=None, slots=None, page_size=0) -> torch.Tensor:
+        """From the stacked down-projection's rows ``proj`` [N, >= q_rank (+ sections)]: the query
+        latent rmsnorm(proj[:, :q_rank]) * q_norm [N, q_rank]; and, with ``kv_rank`` > 0, each token's
+        page row [rmsnorm(proj[:, kv_col : kv_col + kv_rank]) * kv_norm | the next rot_dim elements turned
+        by the token's position] written at its slot of ``pages`` [pages, 1, page_size, kv_rank + rot_dim]."""
+        self._rows(proj, "latent_prepare input")
+        n = proj.shape[0]
+        if proj.dtype != act_dtype:
+            raise KernelError("latent_prepare: the projection comes in the activation dtype")
+        if q_norm.numel() != q_rank or not q_norm.is_contiguous():
+            raise KernelError("latent_prepare: the query latent's norm weight does not fit")
+        c_q = torch.empty((n, q_rank), dtype=act_dtype, device=proj.device)
+        cos = sin = None
+        max_pos = inter = 0
+        if kv_rank:
+            if kv_norm is None or kv_norm.numel() != kv_rank or kv_norm.dtype != q_norm.dtype or not kv_norm.is_contiguous():
+                raise KernelError("latent_prepare: the latent's norm weight does not fit")
+            if pages is None or pages.dtype != act_dtype or not pages.is_contiguous() or pages.dim() != 4 or pages.shape[1] != 1 \
+                    or pages.shape[2] != page_size or pages.shape[3] != kv_rank + rot_dim:
+                raise KernelError(f"latent_prepare: pages {None if pages is None else tuple(pages.shape)} do not hold rows of {kv_rank + rot_dim}")
+            if rot_dim:
+                if rotation is None or rotation.rotary_dim != rot_dim:
+                    raise KernelError("latent_prepare: the rotation must cover the rotated part exactly")
+                cos, sin, max_pos, inter = rotation.cos, rotation.sin, rotation.cos.shape[0], int(rotation.interleaved)
+        self._check(self.lib.yk_latent_prepare(
+            proj.data_ptr(), proj.stride(0), _code(proj.dtype), q_rank, q_norm.data_ptr(), _code(q_norm.dtype), float(eps),
+            c_q.data_ptr(), kv_col, kv_rank, rot_dim, _ptr(kv_norm), _ptr(positions), _ptr(cos), _ptr(sin), inter, max_pos,
+            _ptr(pages) if kv_rank else None, _ptr(slots) if kv_rank else None, n, self._stream()))
+        return c_q
+
+    def head_linear(self, x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0):
+        """Per head, out[n, h, :out_dim] = x[n, h, :in_dim] . w[h] with w [heads, in_dim, out_dim]
+        (float32 sums).  ``tail`` further elements of every head of x follow the product in the output,
+        turned by the token's position (``rotation``, ``positions``); ``gate`` [N, >= gate_col + heads]:
+        head h's output is multiplied by sigmoid(gate[n, gate_col + h])."""
+        self._rows(x, "head_linear input")
+        n = x.shape[0]
+        if tuple(w.shape) != (n_heads, in_dim, out_dim) or not w.is_contiguous() or x.shape[1] != n_heads * (in_dim + tail):
+            raise KernelError(f"head_linear: input {tuple(x.shape)} and weight {tuple(w.shape)} do not fit {n_heads} heads of {in_dim} (+{tail}) -> {out_dim}")
+        out = torch.empty((n, n_heads * (out_dim + tail)), dtype=out_dtype, device=x.device)
+        if gate is not None:
+            self._rows(gate, "head_linear gate")
+            if gate.shape[0] != n or gate.shape[1] < gate_col + n_heads:
+                raise KernelError("head_linear: the gate's rows do not hold a column per head")
+        if x.dtype == torch.float32 and tail == 0 and (gate is None or gate.dtype == out_dtype):
+            self._check(self.lib.yk_head_linear_out(
+                x.data_ptr(), x.stride(0), w.data_ptr(), _code(w.dtype), out.data_ptr(), _code(out_dtype), n_heads, in_dim, out_dim,
+                _ptr(gate), 0 if gate is None else gate.stride(0), gate_col, n, self._stream()))
+            return out
+        cos = sin = None
+        inter = 0
+        if tail:
+            if rotation is None or rotation.rotary_dim != tail or positions is None:
+                raise KernelError("head_linear: the tail needs a rotation that covers it exactly, and positions")
+            cos, sin, inter = rotation.cos, rotation.sin, int(rotation.interleaved)
+        if gate is not None and gate.dtype != x.dtype:
+            raise KernelError("head_linear: gate and input differ in dtype")
+        self._check(self.lib.yk_head_linear(
+            x.data_ptr(), x.stride(0), _code(x.dtype), w.data_ptr(), _code(w.dtype), out.data_ptr(), _code(out_dtype), n_heads, in_dim,
+            out_dim, tail, _ptr(positions), _ptr(cos), _ptr(sin), inter, _ptr(gate), 0 if gate is None else gate.stride(0), gate_col,
+            n, self._stream()))
+        return out
+
+    def latent_tile_tokens(self, n_heads: int) -> int:
+        """Consecutive tokens of a request that one workgroup of ``latent_attention`` takes."""
+        return self._ask("yk_latent_tile_tokens", n_heads)
+
+    def latent_attention(self, q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None) -> torch.Tensor:
+        """Causal softmax attention of ``q_lat`` (float32 [N, heads * (kv_rank + rot_dim)]) over the page
+        rows [c | kr] of each token's request: scores q . row * scale, the result sum_j p_j c_j as
+        float32 [N, heads * kv_rank].  ``tiles``: the step's spans cut into ``latent_tile_tokens`` tokens
+        (rows of request, first token, count, first position)."""
+        n = q_lat.shape[0]
+        width = kv_rank + rot_dim
+        if q_lat.dtype != torch.float32 or not q_lat.is_contiguous() or q_lat.shape[1] != n_heads * width:
+            raise KernelError("latent_attention: queries are contiguous float32 [N, heads * (kv_rank + rot_dim)]")
+        if pages.dim() != 4 or pages.shape[1] != 1 or pages.shape[2] != page_size or pages.shape[3] != width or not pages.is_contiguous():
+            raise KernelError(f"latent_attention: pages {tuple(pages.shape)} do not hold rows of {width}")
+        if tiles is None:
+            tiles = ctx.arrays[f"latent_tiles_{self.latent_tile_tokens(n_heads)}"]
+        bt = ctx.arrays[f"block_table_g{group}"]
+        out = torch.empty((n, n_heads * kv_rank), dtype=torch.float32, device=q_lat.device)
+        self._check(self.lib.yk_latent_attention(
+            q_lat.data_ptr(), pages.data_ptr(), _code(pages.dtype), tiles.data_ptr(), tiles.shape[0], bt.data_ptr(), bt.shape[1],
+            page_size, n_heads, kv_rank, rot_dim, float(scale), out.data_ptr(), self._stream()))
+        return out
+
+    # ---------------------------------------------------------------- a matrix per head as the memory
+    def conv_state_push(self, x, state, ctx) -> None:
+        """``state`` [slots, keep, channels] (a request's last inputs of a convolution, oldest first)
+        takes in each request's span of ``x`` [N, channels]."""
+        n, channels = x.shape
+        if x.stride(1) != 1 or state.dtype != x.dtype or state.dim() != 3 or state.shape[2] != channels or not state.is_contiguous():
+            raise KernelError("conv_state_push: the state does not match the inputs")
+        a = ctx.arrays
+        self._check(self.lib.yk_conv_state_push(
+            x.data_ptr(), x.stride(0), _code(x.dtype), state.data_ptr(), a["seq_qstart"].data_ptr(), a["seq_qlen"].data_ptr(),
+            a["state_slots"].data_ptr(), a["seq_qstart"].numel(), state.shape[1], channels, self._stream()))
+
+    def linear_state_scan(self, qkv, n_heads, n_kv, dim, vdim, state, ctx, q_scale=1.0, unit_eps=None, decay=None, beta=None):
+        """The recurrence S <- diag(a) S; u = v or beta (v - S^T k); S += k u^T; o = S^T q over each
+        request's span, S [slots, heads, dim, vdim] float32 updated in place.  ``qkv`` [N, >= 2 * kv_heads *
+        dim + heads * vdim]: columns [q | k | v].  ``unit_eps``: q and k are divided by sqrt(sum of squares +
+        unit_eps) first; q is multiplied by ``q_scale``.  ``decay``: ("head", x, col, A_log, dt_bias): a =
+        exp(-exp(A_log) softplus(x[:, col + h] + dt_bias)); ("channel", z, col, bias, tau): a_i = sigmoid(z[:,
+        col + h * dim + i] + bias)^(1 / tau); x, z float32.  ``beta``: (x, col) -> sigmoid(x[:, col + h]), or
+        None for plain writes.  Returns o float32 [N, heads * vdim]."""
+        self._rows(qkv, "linear_state_scan input")
+        n = qkv.shape[0]
+        if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (n_heads, dim, vdim):
+            raise KernelError(f"linear_state_scan: state {tuple(state.shape)} does not hold {n_heads} matrices of {dim} x {vdim}")
+        kind, src, col = decay[0], decay[1], int(decay[2])
+        need = n_heads if kind == "head" else n_heads * dim
+        for t, what, cols in ((src, "decay", col + need),) + (((beta[0], "beta", int(beta[1]) + n_heads),) if beta is not None else ()):
+            if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or t.shape[0] != n or t.shape[1] < cols:
+                raise KernelError(f"linear_state_scan: the {what}'s input must be float32 rows of at least {cols} columns")
+        if kind == "head":
+            p0, p1, tau = decay[3], decay[4], 1.0
+            ok = all(p.dtype == torch.float32 and p.numel() == n_heads and p.is_contiguous() for p in (p0, p1))
+        elif kind == "channel":
+            p0, p1, tau = decay[3], None, float(decay[4])
+            ok = p0.dtype == torch.float32 and p0.numel() == n_heads * dim and p0.is_contiguous()
+        else:
+            raise KernelError(f"linear_state_scan: unknown kind of decay {kind!r}")
+        if not ok:
+            raise KernelError("linear_state_scan: the decay's constants must be contiguous float32 of the heads' size")
+        a = ctx.arrays
+        out = torch.empty((n, n_heads * vdim), dtype=torch.float32, device=qkv.device)
+        self._check(self.lib.yk_linear_state_scan(
+            qkv.data_ptr(), qkv.stride(0), _code(qkv.dtype), n_heads, n_kv, dim, vdim, state.data_ptr(), a["seq_qstart"].data_ptr(),
+            a["seq_qlen"].data_ptr(), a["state_slots"].data_ptr(), a["seq_qstart"].numel(), float(q_scale),
+            -1.0 if unit_eps is None else float(unit_eps), 0 if kind == "head" else 1, src.data_ptr(), src.stride(0), col,
+            p0.data_ptr(), _ptr(p1), tau, None if beta is None else beta[0].data_ptr(), 0 if beta is None else beta[0].stride(0),
+            0 if beta is None else int(beta[1]), out.data_ptr(), self._stream()))
+        return out
+
+    def gated_head_norm(self, o, weight, eps, gate, gate_col, n_heads, vdim, out_dtype) -> torch.Tensor:
+        """Per head, o / sqrt(mean(o^2) + eps) * weight * silu(gate[:, gate_col + h * vdim + .]); ``o`` float32
+        [N, heads * vdim], ``weight`` [vdim] shared by the heads."""
+        n = o.shape[0]
+        self._rows(gate, "gated_head_norm gate")
+        if o.dtype != torch.float32 or not o.is_contiguous() or o.shape[1] != n_heads * vdim or weight.numel() != vdim or not weight.is_contiguous():
+            raise KernelError("gated_head_norm: o is contiguous float32 [N, heads * vdim], the weight [vdim]")
+        if gate.dtype != out_dtype or gate.shape[0] != n or gate.shape[1] < gate_col + n_heads * vdim:
+            raise KernelError("gated_head_norm: the gate does not fit")
+        out = torch.empty((n, n_heads * vdim), dtype=out_dtype, device=o.device)
+        self._check(self.lib.yk_gated_head_norm(
+            o.data_ptr(), weight.data_ptr(), _code(weight.dtype), float(eps), gate.data_ptr(), _code(gate.dtype), gate.stride(0),
+            gate_col, n_heads, vdim, out.data_ptr(), _code(out_dtype), n, self._stream()))
         return out
 
     # spans of more than this many tokens are scanned in chunks (cut by the caller)

@@ -86,6 +86,20 @@ class Settled:
         self.activations = activations
 
 
+class NormedBranch:
+    """A pending contribution that joins the residual through a norm of its own:
+    ``residual += scale * norm(branch)``.  A block that norms its branches' outputs hands the last
+    one on in this form, so that whoever norms the stream next (the next block's first norm, the
+    final norm on the wanted rows) can add it in the same pass; ``settle`` adds it for whoever
+    cannot."""
+
+    def __init__(self, branch, norm: "Norm", scale: float = 1.0):
+        self.branch, self.norm, self.scale = branch, norm, float(scale)
+
+    def settle(self, residual: torch.Tensor) -> None:
+        self.norm.norm_add(residual, self.branch, scale=self.scale)
+
+
 class Part:
     """Common to all parts."""
 
@@ -184,8 +198,8 @@ class Norm(Part):
         """The same on the rows ``rows`` only, without changing ``residual``."""
         raise NotImplementedError
 
-    def norm_add(self, residual: torch.Tensor, branch, expert_rows=None, expert_weight: float = 1.0) -> torch.Tensor:
-        """residual (float32, in place) += norm(branch): a branch's output is normed on its way into
+    def norm_add(self, residual: torch.Tensor, branch, expert_rows=None, expert_weight: float = 1.0, scale: float = 1.0) -> torch.Tensor:
+        """residual (float32, in place) += scale * norm(branch): a branch's output is normed on its way into
         the stream.  ``branch`` is whatever a part's ``forward`` returned, and / or the uncombined rows
         of a mixture of experts (``FeedForward.forward`` may return an ``ExpertRows``).  Returns the
         new residual in the activation dtype."""

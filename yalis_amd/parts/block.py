@@ -11,7 +11,7 @@ returns its own last contribution, to be added by whoever comes next.
 """
 from __future__ import annotations
 
-from .base import Block, Settled, register_block
+from .base import Block, NormedBranch, Settled, register_block
 
 
 @register_block("prenorm")
@@ -76,3 +76,39 @@ class BranchNormBlock(Block):
         if self.feed_forward is not None:
             h = self.feed_forward_norm.norm_add(residual, self.feed_forward.forward(h, ctx))
         return Settled(h)
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """Norms before and after every branch, and a multiplier on what the branches add:
+    x = x + s * post_1(mixer(pre_1(x))); x = x + s * post_2(feed_forward(pre_2(x))).
+    A layer may leave the feed-forward (and its two norms) out.  ``branch_scale`` is s.
+
+    Between two branches the stream is touched once: the norm that reads it next adds the pending
+    branch (through that branch's own norm, scaled) and norms the sum in the same pass.  The last
+    branch is handed on the same way (``NormedBranch``) to whatever norms the stream next."""
+
+    roles = {
+        "mixer_norm": ("norm", True),
+        "mixer": ("mixer", True),
+        "mixer_out_norm": ("norm", True),
+        "feed_forward_norm": ("norm", False),
+        "feed_forward": ("feed_forward", False),
+        "feed_forward_out_norm": ("norm", False),
+    }
+
+    def __init__(self, mixer_norm, mixer, mixer_out_norm, feed_forward_norm=None, feed_forward=None, feed_forward_out_norm=None,
+                 branch_scale: float = 1.0):
+        if len({feed_forward is None, feed_forward_norm is None, feed_forward_out_norm is None}) != 1:
+            raise ValueError("a sandwich block has a feed-forward with both of its norms, or none of the three")
+        self.mixer_norm, self.mixer, self.mixer_out_norm = mixer_norm, mixer, mixer_out_norm
+        self.feed_forward_norm, self.feed_forward, self.feed_forward_out_norm = feed_forward_norm, feed_forward, feed_forward_out_norm
+        self.branch_scale = float(branch_scale)
+
+    def forward(self, residual, delta, ctx, site):
+        h = self.mixer_norm.add_norm(residual, delta)
+        pending = NormedBranch(self.mixer.forward(h, ctx, site), self.mixer_out_norm, self.branch_scale)
+        if self.feed_forward is None:
+            return pending
+        h = self.feed_forward_norm.add_norm(residual, pending)
+        return NormedBranch(self.feed_forward.forward(h, ctx), self.feed_forward_out_norm, self.branch_scale)

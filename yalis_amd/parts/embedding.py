@@ -53,7 +53,7 @@ class TokenEmbedding(Part):
 @register_head("lm_head")
 class LMHead(Part):
     """params: name, tied_to (name of the embedding table, or None), vocab_size,
-    hidden_size."""
+    hidden_size, scale (1.0: what the logits are multiplied with)."""
 
     graph_capturable = True
 
@@ -63,6 +63,7 @@ class LMHead(Part):
         self.tied_to = params.get("tied_to")
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
+        self.scale = float(params.get("scale", 1.0))
         self.weight = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -83,4 +84,7 @@ class LMHead(Part):
         return ((self.vocab, self.hidden),)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return self.rt.ops.linear(h, self.weight, torch.float32)
+        logits = self.rt.ops.linear(h, self.weight, torch.float32)
+        if self.scale != 1.0:
+            self.rt.ops.scale_rows(logits, self.scale)
+        return logits

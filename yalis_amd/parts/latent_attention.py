@@ -1,0 +1,146 @@
+"""Causal attention whose keys and values come from one small latent per token.
+
+For a token with mixer input h and position p, per head (dim unrotated, rot_dim rotated query and
+key elements, value_dim value elements):
+    c_q = rmsnorm(W_dq h) * w_dq          q = W_uq c_q, head by head [dim | rot_dim]
+    [l ; r] = W_dkv h                     c = rmsnorm(l) * w_dkv  (kv_rank)    kr = turn(r, p)  (rot_dim, one for all heads)
+    k_head = W_uk,head c                  v_head = W_uv,head c
+    score(i, j) = (q_i[:dim] . k_head,j + turn(q_i[dim:], i) . kr_j) * scale,  softmax over j <= i
+    out = W_o concat_heads(sigmoid(W_g h)_head * sum_j p_ij v_head,j)
+A token's page row holds [c | kr] and nothing else; a layer may read another layer's pages
+(``RunEntry.cache_from``) with W_uk, W_uv and queries of its own.
+
+The up-projections never touch the cached rows: since q[:dim] . (W_uk c) = (W_uk^T q[:dim]) . c and
+sum_j p_j W_uv c_j = W_uv sum_j p_j c_j, the queries are taken into the latent's space once per
+token ([W_uk^T q[:dim] | turned q[dim:]], float32), the attention runs over the page rows as they
+are, with one shared "key" of kv_rank + rot_dim elements and the latent itself as the value, and
+W_uv is applied to the kv_rank-wide result of each head.
+
+params: prefix, hidden_size, num_heads, head_dim, rot_dim, value_dim, kv_rank, q_rank, scale,
+latent_eps (of the two latent norms), gate (tensor name below the prefix or None), position (a
+PartSpec whose ``rotation()`` covers exactly rot_dim elements), names (optional overrides).
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping
+
+import torch
+
+from ..config.specs import PartSpec
+from ..engine.batch import attention_tiles
+from ..weights.loader import TensorSpec
+from .base import POSITIONS, KVNeed, Mixer, Runtime, register_mixer
+
+
+def _pad_rows(parts, multiple: int):
+    rows = sum(p.shape[0] for p in parts)
+    pad = -rows % multiple
+    if pad:
+        parts = list(parts) + [torch.zeros((pad, parts[0].shape[1]), dtype=parts[0].dtype, device=parts[0].device)]
+    return torch.cat(list(parts), dim=0).contiguous()
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    graph_capturable = True
+
+    def __init__(self, params, rt: Runtime):
+        super().__init__(params, rt)
+        self.prefix = params["prefix"]
+        self.hidden = int(params["hidden_size"])
+        self.n_heads = int(params["num_heads"])
+        self.head_dim = int(params["head_dim"])
+        self.rot_dim = int(params["rot_dim"])
+        self.value_dim = int(params["value_dim"])
+        self.kv_rank = int(params["kv_rank"])
+        self.q_rank = int(params["q_rank"])
+        self.scale = float(params["scale"])
+        self.eps = float(params["latent_eps"])
+        self.gate_name = params.get("gate")
+        self.projects_kv = bool(params.get("projects_kv", True))
+        pos: PartSpec = params["position"]
+        self.position = POSITIONS.get(pos.kind)(pos.params, rt)
+        self.rotation = self.position.rotation()
+        if self.rotation is None or self.rotation.rotary_dim != self.rot_dim:
+            raise ValueError(f"{self.prefix}: the position encoding must rotate exactly the rot_dim={self.rot_dim} elements of the rotated part")
+        names = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o"}
+        names.update(params.get("names", {}))
+        self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
+        self.w_down = self.w_qn = self.w_kvn = self.w_uq = self.w_uk = self.w_uv_t = self.w_o = None
+        # columns of the stacked down-projection: [dq | dkv (where the layer keeps a cache) | gates], each
+        # section starting at a multiple of 8
+        up8 = lambda n: n + (-n % 8)
+        self.kv_col = up8(self.q_rank)
+        self.gate_col = self.kv_col + (up8(self.kv_rank + self.rot_dim) if self.projects_kv else 0)
+        self.down_rows = self.gate_col + (self.n_heads if self.gate_name else 0)
+        self.down_rows += -self.down_rows % 16
+        # consecutive tokens of a request that one workgroup of the attention takes
+        self.tile_tokens = int(rt.ops.latent_tile_tokens(self.n_heads))
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, H = self.names, self.n_heads
+        specs = {
+            n["dq"]: TensorSpec((self.q_rank, self.hidden)), n["dq_norm"]: TensorSpec((self.q_rank,), "float", ("one_plus_normal", 0.1)),
+            n["uq"]: TensorSpec((H * (self.head_dim + self.rot_dim), self.q_rank)),
+            n["uk"]: TensorSpec((H * self.head_dim, self.kv_rank)), n["uv"]: TensorSpec((H * self.value_dim, self.kv_rank)),
+            n["o"]: TensorSpec((self.hidden, H * self.value_dim)),
+        }
+        if self.projects_kv:
+            specs[n["dkv"]] = TensorSpec((self.kv_rank + self.rot_dim, self.hidden))
+            specs[n["dkv_norm"]] = TensorSpec((self.kv_rank,), "float", ("one_plus_normal", 0.1))
+        if self.gate_name:
+            specs[f"{self.prefix}.{self.gate_name}"] = TensorSpec((H, self.hidden))
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        n, H = self.names, self.n_heads
+        dq = tensors[n["dq"]]
+        zeros = lambda rows: torch.zeros((rows, self.hidden), dtype=dq.dtype, device=dq.device)
+        parts = [dq, zeros(self.kv_col - self.q_rank)]
+        if self.projects_kv:
+            parts += [tensors[n["dkv"]], zeros(self.gate_col - self.kv_col - self.kv_rank - self.rot_dim)]
+            self.w_kvn = tensors[n["dkv_norm"]].contiguous()
+        if self.gate_name:
+            parts.append(tensors[f"{self.prefix}.{self.gate_name}"])
+        parts.append(zeros(self.down_rows - sum(p.shape[0] for p in parts)))
+        self.w_down = torch.cat([p for p in parts if p.shape[0]], dim=0).contiguous()
+        self.w_qn = tensors[n["dq_norm"]].contiguous()
+        self.w_uq = tensors[n["uq"]]
+        # per head [in][out]: W_uk as it is stored ([head][dim][kv_rank]: out = kv_rank), W_uv transposed
+        # ([head][kv_rank][value_dim])
+        self.w_uk = tensors[n["uk"]].view(H, self.head_dim, self.kv_rank).contiguous()
+        self.w_uv_t = tensors[n["uv"]].view(H, self.value_dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_o = tensors[n["o"]]
+
+    def kv_need(self) -> KVNeed:
+        # one row of kv_rank + rot_dim elements per token and no values: the row serves as both
+        return KVNeed(1, self.kv_rank + self.rot_dim, None, 0)
+
+    def products(self):
+        H = self.n_heads
+        return ((self.down_rows, self.hidden), (H * (self.head_dim + self.rot_dim), self.q_rank), (self.hidden, H * self.value_dim))
+
+    def step_inputs(self):
+        n = self.tile_tokens
+        return {f"latent_tiles_{n}": lambda hb: attention_tiles(hb, n)}
+
+    def forward(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
+        ops, act = self.rt.ops, self.rt.act_dtype
+        if site.owns_cache != self.projects_kv:
+            raise RuntimeError(f"{self.prefix}: a layer whose run entries both own and borrow caches is not offered")
+        proj = ops.linear(h, self.w_down, act)
+        pages, _ = site.kv()
+        c_q = ops.latent_prepare(
+            proj, self.q_rank, self.w_qn, self.eps, act, kv_col=self.kv_col, kv_rank=self.kv_rank if site.owns_cache else 0,
+            rot_dim=self.rot_dim, kv_norm=self.w_kvn, rotation=self.rotation, positions=ctx.arrays["positions"], pages=pages,
+            slots=ctx.arrays[f"slots_g{site.group}"], page_size=self.rt.page_size,
+        )
+        q = ops.linear(c_q, self.w_uq, act)
+        # queries in the latent's space: [W_uk^T q[:dim] | q[dim:] turned by the position], float32
+        q_lat = ops.head_linear(q, self.w_uk, self.n_heads, self.head_dim, self.kv_rank, torch.float32, tail=self.rot_dim,
+                                rotation=self.rotation, positions=ctx.arrays["positions"])
+        o_lat = ops.latent_attention(q_lat, pages, self.n_heads, self.kv_rank, self.rot_dim, self.scale, ctx, site.group,
+                                     self.rt.page_size, tiles=ctx.arrays[f"latent_tiles_{self.tile_tokens}"])
+        o = ops.head_linear(o_lat, self.w_uv_t, self.n_heads, self.kv_rank, self.value_dim, act,
+                            gate=proj if self.gate_name else None, gate_col=self.gate_col)
+        return ops.linear(o, self.w_o, act, partial_ok=True)

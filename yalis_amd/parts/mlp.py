@@ -20,6 +20,7 @@ from ..weights.loader import TensorSpec
 from .base import FeedForward, Runtime, register_feed_forward
 
 ACTIVATIONS = ("silu", "gelu_tanh")
+DENSE_ACTIVATIONS = ("relu2", "silu", "gelu_tanh")
 
 
 @register_feed_forward("gated_mlp")
@@ -78,4 +79,41 @@ class GatedMLP(FeedForward):
             a = ops.gated_act(torch.cat([gate, up], dim=1), self.activation, self.rt.act_dtype)
             return ops.linear(a, self.w_down, self.rt.act_dtype, bias=self.b_down)
         a = ops.gate_up_act(h, self.w_gate_up, self.gate_up_group, self.activation, self.rt.act_dtype)
+        return ops.linear(a, self.w_down, self.rt.act_dtype, partial_ok=True)
+
+
+@register_feed_forward("dense_mlp")
+class DenseMLP(FeedForward):
+    """down(act(up h)), no gate, no biases.
+
+    params: prefix, hidden_size, intermediate_size, activation ("relu2": the square of relu; "silu",
+    "gelu_tanh"), names (optional overrides of the two tensor names below the prefix)."""
+
+    graph_capturable = True
+
+    def __init__(self, params, rt: Runtime):
+        super().__init__(params, rt)
+        self.prefix = params["prefix"]
+        self.hidden = int(params["hidden_size"])
+        self.inter = int(params["intermediate_size"])
+        self.activation = params.get("activation", "relu2")
+        if self.activation not in DENSE_ACTIVATIONS:
+            raise ValueError(f"activation {self.activation!r} is not supported (supported: {DENSE_ACTIVATIONS})")
+        names = {"up": "up_proj.weight", "down": "down_proj.weight"}
+        names.update(params.get("names", {}))
+        self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
+        self.w_up = self.w_down = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.names["up"]: TensorSpec((self.inter, self.hidden)), self.names["down"]: TensorSpec((self.hidden, self.inter))}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_up, self.w_down = tensors[self.names["up"]], tensors[self.names["down"]]
+
+    def products(self):
+        return ((self.inter, self.hidden), (self.hidden, self.inter))
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        ops = self.rt.ops
+        a = ops.activation(ops.linear(h, self.w_up, self.rt.act_dtype, partial_ok=True), self.activation, self.rt.act_dtype)
         return ops.linear(a, self.w_down, self.rt.act_dtype, partial_ok=True)

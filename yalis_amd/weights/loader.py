@@ -45,6 +45,12 @@ class TensorSpec:
     shape: Tuple[int, ...]
     kind: str = "float"
     init: Tuple = ("normal", 0.02)
+    # axes whose length the checkpoint decides (``shape`` holds what the random-weights mode makes)
+    free_axes: Tuple[int, ...] = ()
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(a == b or i in self.free_axes for i, (a, b) in enumerate(zip(shape, self.shape)))
 
 
 class WeightsError(RuntimeError):
@@ -105,7 +111,7 @@ def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec]
     wrong_shape = [
         (n, entries[n].shape, s.shape)
         for n, s in wanted.items()
-        if n in entries and tuple(entries[n].shape) != tuple(s.shape)
+        if n in entries and not s.fits(entries[n].shape)
     ]
     wrong_kind = []
     for n, s in wanted.items():
