@@ -29,6 +29,9 @@ each with the fraction of the peak that bounds it.
 of the Suranex design at two layer sizes beside the Llama configuration of equal width, depth, heads
 and active feed-forward width, one JSON line a size, with the time of every kind of call into the
 kernel library, its bound max(bytes / 8 TB/s, flops / 2.5 PFLOP/s) and time / bound.
+``--design nutavik`` does the same for the Nutavik design (latent attention, delta rule, gated linear
+attention, dense feed-forward) beside the Llama configuration of equal width, depth, heads and
+feed-forward weights.
 """
 import argparse
 import json
@@ -425,12 +428,28 @@ def _op_costs(ops, hb):
         u, wa = a[0], a[3]
         return 4.0 * u.shape[0] * u.shape[1] * wa.shape[1], nbytes(u) * 4 + nbytes(wa) * 2
 
+    def head_linear(a, kw, out):
+        x, w = a[0], a[1]
+        return 2.0 * x.shape[0] * w.numel(), float(nbytes(x, w, out))
+
+    def latent_attention(a, kw, out):
+        q, pages, heads, rank, rot = a[0], a[1], a[2], a[3], a[4]
+        b = hb()
+        return 2.0 * heads * (2 * rank + rot) * visible(0, 0), float(pages.element_size() * (rank + rot) * sum(b.seq_ctx.tolist()) + nbytes(q, out))
+
+    def state_scan(a, kw, out):
+        qkv, heads, dim, vdim, state = a[0], a[1], a[3], a[4], a[5]
+        b = hb()
+        return 6.0 * qkv.shape[0] * heads * dim * vdim, float(nbytes(qkv, out) + 8.0 * b.n_seqs * heads * dim * vdim)
+
     def moved(a, kw, out):
         return 0.0, float(nbytes(*a, *kw.values()) + (nbytes(out) if hasattr(out, "numel") else 0))
 
     return {"linear": linear, "gate_up_act": linear, "moe_experts": moe, "attention_masked": attention_masked, "attention": attention,
             "rglru": rglru, "norm_add": moved, "add_rmsnorm": moved, "gather_add_rmsnorm": moved, "qkv_prepare": moved,
-            "rope_append": moved, "causal_conv": moved, "gated_act": moved, "round_rows": moved, "embed": moved}
+            "rope_append": moved, "causal_conv": moved, "gated_act": moved, "round_rows": moved, "embed": moved,
+            "sandwich_norm": moved, "activation": moved, "latent_prepare": moved, "head_linear": head_linear,
+            "latent_attention": latent_attention, "linear_state_scan": state_scan, "gated_head_norm": moved, "conv_state_push": moved}
 
 
 def per_op_times(runner, vocab: int, gen, batch: int, prompt_len: int, prefill_len: int):
@@ -522,7 +541,7 @@ def design_compare(args) -> int:
 
     from yalis_amd.models.presets import llama_like
 
-    sizes = {"suranex": ("suranex-2k", "suranex-4k")}[args.design]
+    sizes = {"suranex": ("suranex-2k", "suranex-4k"), "nutavik": ("nutavik-2k", "nutavik-4k")}[args.design]
     if args.design_shape:
         sizes = (args.design_shape,)
     for name in sizes:
@@ -551,9 +570,9 @@ def design_compare(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=("suranex",), default=None,
+    ap.add_argument("--design", choices=("suranex", "nutavik"), default=None,
                     help="measure instead another design's prefill and decode at a few layer sizes, beside the Llama configuration of equal size, with the time and the bound of every kind of kernel")
-    ap.add_argument("--design-shape", default=None, help="with --design: one of its shapes only (suranex-2k, suranex-4k)")
+    ap.add_argument("--design-shape", default=None, help="with --design: one of its shapes only (suranex-2k, suranex-4k, nutavik-2k, nutavik-4k)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=32)
     ap.add_argument("--warmup", type=int, default=4)

@@ -97,7 +97,9 @@ class NutavikConfig:
     def _gla(m: Dict[str, Any], where: str) -> Dict[str, Any]:
         r = KeyReader(m, where=where)
         out = {"heads": r.integer("heads", minimum=1), "dim": r.integer("dim", minimum=1), "vdim": r.integer("vdim", minimum=1),
-               "tau": r.number("tau", positive=True)}
+               "tau": r.number("tau", positive=True),
+               # the rank of the decay's pair of projections: read from the tensors' shapes unless given
+               "low_rank": r.integer("low_rank", default=None, minimum=1)}
         r.finish()
         return out
 
@@ -168,7 +170,8 @@ def build_nutavik_spec(cfg: NutavikConfig) -> ModelSpec:
                 unit_eps=UNIT_EPS, out_norm_eps=cfg.eps))
         else:
             mixer = PartSpec("gated_linear_attention", dict(
-                common, num_heads=m["heads"], head_dim=m["dim"], value_dim=m["vdim"], tau=m["tau"], out_norm_eps=cfg.eps))
+                common, num_heads=m["heads"], head_dim=m["dim"], value_dim=m["vdim"], tau=m["tau"], low_rank=m["low_rank"],
+                out_norm_eps=cfg.eps))
         ffn = ffn_norm = ffn_out = None
         if layer.mlp is not None:
             ffn = PartSpec("dense_mlp", {"prefix": f"{p}.mlp", "hidden_size": cfg.width, "intermediate_size": layer.mlp["ff"],

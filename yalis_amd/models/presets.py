@@ -61,10 +61,39 @@ def suranex_shape(width: int, vocab: int, heads: int, kv_heads: int, dim: int, w
     return {"architecture": "Suranex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": layers}
 
 
-def llama_like(suranex: dict) -> dict:
-    """The Llama configuration of equal size: the same width, layer count, vocabulary and (first
-    attention layer's) heads, a feed-forward as wide as what a token uses of the mixture (its top
-    experts and the shared one)."""
+def nutavik_shape(width: int, vocab: int, heads: int, dim: int, rot_dim: int, kv_rank: int, q_rank: int, delta_heads: int,
+                  delta_kv_heads: int, gla_heads: int, gla_dim: int, gla_vdim: int, ff: int, repeats: int = 2) -> dict:
+    """A Nutavik config.json of the given layer sizes: (latent attention, delta rule, gated linear
+    attention) repeated ``repeats`` times, every layer with a dense feed-forward; latent-attention
+    layers after the first read the first one's cache."""
+    rot = {"base": 10000.0, "dims": rot_dim, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    att = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": dim, "kv_rank": kv_rank, "q_rank": q_rank,
+           "scale": (dim + rot_dim) ** -0.5, "rot": rot}
+    dl = {"heads": delta_heads, "kv_heads": delta_kv_heads, "dim": dim, "vdim": dim, "conv": 4}
+    gl = {"heads": gla_heads, "dim": gla_dim, "vdim": gla_vdim, "tau": 16.0, "low_rank": 16}
+    layers = []
+    for r in range(repeats):
+        layers.append({"type": "latent_attention", "mixer": dict(att, **({"kv_from": 0} if r else {})), "mlp": {"kind": "dense", "ff": ff}})
+        layers.append({"type": "delta", "mixer": dict(dl), "mlp": {"kind": "dense", "ff": ff}})
+        layers.append({"type": "gla", "mixer": dict(gl), "mlp": {"kind": "dense", "ff": ff}})
+    return {"architecture": "Nutavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5, "logit_scale": 1.0,
+            "layers": layers}
+
+
+def llama_like(design: dict) -> dict:
+    """The Llama configuration of equal size.  For Suranex: the same width, layer count, vocabulary
+    and (first attention layer's) heads, a feed-forward as wide as what a token uses of the mixture
+    (its top experts and the shared one).  For Nutavik: the same width, layer count, vocabulary and
+    attention heads (keys as wide as its unrotated and rotated parts together, a quarter as many key
+    heads), a gated feed-forward with as many weights as its dense one (two thirds as wide)."""
+    if design.get("architecture") == "Nutavik":
+        att = next(layer["mixer"] for layer in design["layers"] if layer["type"] == "latent_attention")
+        ff = next(layer["mlp"]["ff"] for layer in design["layers"] if layer["mlp"] is not None)
+        head_dim = 128 if att["dim"] + att["rot_dim"] > 64 else 64
+        return dict(LLAMA3_8B, hidden_size=design["width"], num_hidden_layers=len(design["layers"]), num_attention_heads=att["heads"],
+                    num_key_value_heads=max(1, att["heads"] // 4), head_dim=head_dim, intermediate_size=(2 * ff // 3 + 255) // 256 * 256,
+                    vocab_size=design["vocab"])
+    suranex = design
     att = next(layer["mixer"] for layer in suranex["layers"] if layer["type"] == "attention")
     mlp = next(layer["mlp"] for layer in suranex["layers"] if layer["mlp"] is not None)
     inter = mlp["router"]["top"] * mlp["expert"]["ff"] + (mlp["shared"]["ff"] if mlp.get("shared") else 0)
@@ -75,6 +104,9 @@ def llama_like(suranex: dict) -> dict:
 SURANEX_2K = suranex_shape(2048, 32768, 16, 4, 128, 1024, 2560, 10, 16, 2, 1024, 2048)
 SURANEX_4K = suranex_shape(4096, 65536, 32, 8, 128, 2048, 5120, 20, 32, 4, 1024, 4096, repeats=1)
 SURANEX_TINY = suranex_shape(64, 256, 4, 2, 16, 24, 96, 3, 4, 2, 32, 48, repeats=1)
+NUTAVIK_2K = nutavik_shape(2048, 32768, 16, 128, 64, 512, 768, 16, 8, 4, 256, 512, 8192)
+NUTAVIK_4K = nutavik_shape(4096, 65536, 32, 128, 64, 512, 1536, 32, 16, 8, 256, 512, 16384, repeats=1)
+NUTAVIK_TINY = nutavik_shape(64, 256, 4, 16, 8, 24, 32, 4, 2, 2, 16, 32, 96, repeats=1)
 
 # name -> (what to call it, config.json dictionary)
 SHAPES: Dict[str, Tuple[str, dict]] = {
@@ -87,6 +119,9 @@ SHAPES: Dict[str, Tuple[str, dict]] = {
     "suranex-2k": ("Suranex, width 2,048", SURANEX_2K),
     "suranex-4k": ("Suranex, width 4,096", SURANEX_4K),
     "suranex-tiny": ("tiny Suranex", SURANEX_TINY),
+    "nutavik-2k": ("Nutavik, width 2,048", NUTAVIK_2K),
+    "nutavik-4k": ("Nutavik, width 4,096", NUTAVIK_4K),
+    "nutavik-tiny": ("tiny Nutavik", NUTAVIK_TINY),
 }
 
 
