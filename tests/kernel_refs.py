@@ -478,7 +478,7 @@ def scale_rows(x, s):
 
 # ------------------------------------------------------------- attention over one latent per token
 def latent_prepare(proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, rot_dim=0, kv_norm=None, rotation=None,
-                   positions=None, pages=None, slots=None, page_size=0):
+                   positions=None, pages=None, slots=None, page_size=0, values=None):
     p = proj.float()
     c_q = _rmsnorm(p[:, :q_rank], q_norm, eps, False).to(act_dtype)
     if kv_rank:
@@ -488,6 +488,8 @@ def latent_prepare(proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, ro
         row = torch.cat([c, r], dim=1).to(pages.dtype)
         s = slots.long()
         pages[s // page_size, 0, s % page_size, :] = row
+        if values is not None:  # the latent once more, transposed
+            values[s // page_size, 0, :, s % page_size] = c.to(values.dtype)
     return c_q
 
 
@@ -507,7 +509,7 @@ def head_linear(x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None
     return out.reshape(n, -1).to(out_dtype)
 
 
-def latent_attention(q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None):
+def latent_attention(q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None, values=None):
     a = ctx.arrays
     n = q_lat.shape[0]
     width = kv_rank + rot_dim
@@ -586,7 +588,8 @@ RefOps.scale_rows = staticmethod(scale_rows)
 RefOps.latent_prepare = staticmethod(latent_prepare)
 RefOps.head_linear = staticmethod(head_linear)
 RefOps.latent_attention = staticmethod(latent_attention)
-RefOps.latent_tile_tokens = staticmethod(lambda n_heads: 16 // min(n_heads, 4))
+RefOps.latent_tile_tokens = staticmethod(lambda n_heads, matrix_cores=False: 16 // min(n_heads, 4))
+RefOps.latent_attention_on_matrix_cores = staticmethod(lambda act_dtype, kv_rank, rot_dim, page_size: False)
 RefOps.causal_conv = staticmethod(causal_conv_act)
 RefOps.conv_state_push = staticmethod(conv_state_push)
 RefOps.linear_state_scan = staticmethod(linear_state_scan)

@@ -40,8 +40,8 @@ def context(spans_at, page, slots=None, tile_tokens=4, device="cuda:0"):
     arrays = {"positions": hb.positions, "token_seq": hb.token_seq, "seq_qstart": hb.seq_qstart, "seq_qlen": hb.seq_qlen,
               "state_slots": hb.state_slots, "block_table_g0": hb.block_tables[0], "slots_g0": hb.slots[0],
               f"latent_tiles_{tile_tokens}": attention_tiles(hb, tile_tokens)}
-    cpu = SimpleNamespace(arrays={k: torch.from_numpy(np.ascontiguousarray(v)) for k, v in arrays.items()})
-    dev = SimpleNamespace(arrays={k: v.to(device) for k, v in cpu.arrays.items()})
+    cpu = SimpleNamespace(arrays={k: torch.from_numpy(np.ascontiguousarray(v)) for k, v in arrays.items()}, max_ctx=hb.max_ctx)
+    dev = SimpleNamespace(arrays={k: v.to(device) for k, v in cpu.arrays.items()}, max_ctx=hb.max_ctx)
     return dev, cpu, n_pages
 
 
@@ -114,13 +114,15 @@ def test_latent_prepare(dtype, q_rank, kv_rank, rot_dim):
     rot = rotation(rot_dim, 64)
     pages_ref = torch.zeros(n_pages, 1, page, kv_rank + rot_dim, dtype=dtype)
     pages_dev = pages_ref.clone().cuda()
+    values_dev = torch.zeros(n_pages, 1, kv_rank, page, dtype=dtype).cuda()
     kw = dict(kv_col=kv_col, kv_rank=kv_rank, rot_dim=rot_dim, page_size=page)
     want = R.latent_prepare(proj, q_rank, qn, 1e-5, dtype, kv_norm=kn, rotation=rot, positions=cpu.arrays["positions"],
                             pages=pages_ref, slots=cpu.arrays["slots_g0"], **kw)
     got = o.latent_prepare(proj.cuda(), q_rank, qn.cuda(), 1e-5, dtype, kv_norm=kn.cuda(), rotation=on_device(rot),
-                           positions=dev.arrays["positions"], pages=pages_dev, slots=dev.arrays["slots_g0"], **kw)
+                           positions=dev.arrays["positions"], pages=pages_dev, slots=dev.arrays["slots_g0"], values=values_dev, **kw)
     close(got, want, dtype, "query latent", bf16=1e-2)
     close(pages_dev, pages_ref, dtype, "page rows", bf16=1e-2)
+    assert torch.equal(values_dev.transpose(2, 3), pages_dev[..., :kv_rank]), "the transposed copy holds the same latents"
     # a layer that reads another's cache writes nothing
     before = pages_dev.clone()
     o.latent_prepare(proj.cuda(), q_rank, qn.cuda(), 1e-5, dtype)
@@ -190,6 +192,50 @@ def test_one_row_stands_out_at_every_border(dtype, heads, kv_rank, rot_dim, spec
     close(got, want.reshape(n_tok, -1), torch.float32, f"row {special}", f32=2e-5)
     seen = [t for t in range(n_tok) if int(pos[t]) >= special]
     if seen:  # where the row is visible it carries nearly all the weight: its own latent comes back
+        assert (got[seen].view(len(seen), heads, kv_rank)[:, :, 0].cpu() > 20.0).all()
+
+
+@pytest.mark.parametrize("heads,kv_rank,rot_dim,page", [(2, 64, 32, 32), (5, 128, 32, 64), (16, 512, 64, 64), (20, 256, 64, 32)])
+@pytest.mark.parametrize("special", [0, 31, 32, 63, 64, 399, 400])
+@pytest.mark.parametrize("splits", [1, 3, None])
+def test_matrix_core_form_at_every_border(heads, kv_rank, rot_dim, page, special, splits):
+    """The same towering row for the matrix-core form (bfloat16 pages, the latent a second time in
+    transposed pages): borders of its groups of 32 keys and of pages, tiles of several tokens where
+    heads are few and of one token's heads in chunks of 16 where they are many, the keys whole,
+    divided in three, and divided as the library decides; against float64 over the same rounded rows."""
+    if kv_rank >= 256 and special not in (0, 63, 64, 400):
+        pytest.skip("the largest sizes run a few of the borders")
+    o = ops()
+    assert o.latent_attention_on_matrix_cores(torch.bfloat16, kv_rank, rot_dim, page)
+    L, width = 700, kv_rank + rot_dim
+    g = torch.Generator().manual_seed(special + heads)
+    rows = torch.randn(L, width, generator=g) * 0.2
+    rows[special, 0] = 30.0
+    rows = rows.to(torch.bfloat16).float()
+    spans_at = [(380, 70), (399, 1), (400, 1), (699, 1), (16, 1)]
+    tile = o.latent_tile_tokens(heads, True)
+    dev, cpu, n_pages = context(spans_at, page, tile_tokens=tile)
+    pages = torch.full((n_pages, 1, page, width), 7.0)  # (slots never written hold something)
+    bt = cpu.arrays["block_table_g0"]
+    for s, (p0, n) in enumerate(spans_at):
+        for j in range(p0 + n):
+            pages[int(bt[s, j // page]), 0, j % page] = rows[j]
+    values = pages[..., :kv_rank].transpose(2, 3).contiguous()
+    n_tok = sum(n for _, n in spans_at)
+    q = (torch.randn(n_tok, heads, width, generator=g) * 0.3)
+    q[:, :, 0] = 1.0
+    q = q.to(torch.bfloat16).float()  # what the kernel rounds its queries to
+    scale = 0.7
+    got = o.latent_attention(q.reshape(n_tok, -1).cuda(), pages.to(torch.bfloat16).cuda(), heads, kv_rank, rot_dim, scale, dev, 0, page,
+                             tiles=dev.arrays[f"latent_tiles_{tile}"], values=values.to(torch.bfloat16).cuda(), splits=splits)
+    pos = cpu.arrays["positions"]
+    want = torch.empty(n_tok, heads, kv_rank, dtype=torch.float64)
+    for t in range(n_tok):
+        keys = rows[: int(pos[t]) + 1].double()
+        want[t] = torch.softmax(q[t].double() @ keys.T * scale, dim=-1) @ keys[:, :kv_rank]
+    close(got, want.reshape(n_tok, -1), torch.bfloat16, f"row {special}", bf16=1e-2)
+    seen = [t for t in range(n_tok) if int(pos[t]) >= special]
+    if seen:
         assert (got[seen].view(len(seen), heads, kv_rank)[:, :, 0].cpu() > 20.0).all()
 
 

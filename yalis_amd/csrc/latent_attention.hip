@@ -25,7 +25,7 @@ __global__ __launch_bounds__(128) void latent_prepare_kernel(
     const T* __restrict__ proj, int proj_stride, int q_rank, const TW* __restrict__ q_norm, float eps, T* __restrict__ c_q,
     int kv_col, int kv_rank, int rot_dim, const TW* __restrict__ kv_norm, const int32_t* __restrict__ positions,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int interleaved, T* __restrict__ pages,
-    const int32_t* __restrict__ slots) {
+    T* __restrict__ pages_t, int page_size, const int32_t* __restrict__ slots) {
   __shared__ float scratch[17];
   const size_t n = blockIdx.x;
   const T* row = proj + n * proj_stride;
@@ -46,8 +46,15 @@ __global__ __launch_bounds__(128) void latent_prepare_kernel(
   }
   inv = 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(kv_rank) + eps);
   T* dst = pages + static_cast<size_t>(slots[n]) * (kv_rank + rot_dim);
-  for (int c = threadIdx.x; c < kv_rank; c += blockDim.x)
-    dst[c] = from_f32<T>(to_f32<T>(kv[c]) * inv * to_f32<TW>(kv_norm[c]));
+  // pages_t: the latent once more, transposed ([page][column][slot]), for readers that want a column's
+  // slots side by side
+  const size_t slot = static_cast<size_t>(slots[n]);
+  T* dst_t = pages_t == nullptr ? nullptr : pages_t + (slot / page_size) * kv_rank * page_size + slot % page_size;
+  for (int c = threadIdx.x; c < kv_rank; c += blockDim.x) {
+    const T v = from_f32<T>(to_f32<T>(kv[c]) * inv * to_f32<TW>(kv_norm[c]));
+    dst[c] = v;
+    if (dst_t != nullptr) dst_t[static_cast<size_t>(c) * page_size] = v;
+  }
   const int half = rot_dim / 2;
   const size_t p = static_cast<size_t>(positions[n]);
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
@@ -62,7 +69,9 @@ __global__ __launch_bounds__(128) void latent_prepare_kernel(
 extern "C" int yk_latent_prepare(const void* proj, int proj_stride, int dtype, int q_rank, const void* q_norm, int w_dtype,
                                  float eps, void* c_q, int kv_col, int kv_rank, int rot_dim, const void* kv_norm,
                                  const int32_t* positions, const float* cos_t, const float* sin_t, int interleaved,
-                                 int max_positions, void* pages, const int32_t* slots, int n_tokens, hipStream_t stream) {
+                                 int max_positions, void* pages, void* pages_t, int page_size, const int32_t* slots,
+                                 int n_tokens, hipStream_t stream) {
+  YK_REQUIRE(pages_t == nullptr || page_size > 0, "latent_prepare: transposed pages need the page size");
   YK_REQUIRE(n_tokens >= 0 && q_rank > 0 && kv_rank >= 0 && rot_dim >= 0 && rot_dim % 2 == 0, "latent_prepare: bad sizes");
   YK_REQUIRE(proj_stride >= q_rank && (kv_rank == 0 || proj_stride >= kv_col + kv_rank + rot_dim),
              "latent_prepare: the projection's rows are shorter than its sections");
@@ -76,7 +85,7 @@ extern "C" int yk_latent_prepare(const void* proj, int proj_stride, int dtype, i
     latent_prepare_kernel<T, TW><<<n_tokens, 128, 0, stream>>>(                                                       \
         static_cast<const T*>(proj), proj_stride, q_rank, static_cast<const TW*>(q_norm), eps, static_cast<T*>(c_q),  \
         kv_col, kv_rank, rot_dim, static_cast<const TW*>(kv_norm), positions, cos_t, sin_t, interleaved,              \
-        static_cast<T*>(pages), slots);                                                                               \
+        static_cast<T*>(pages), static_cast<T*>(pages_t), page_size, slots);                                          \
     return yk_check_launch("latent_prepare");                                                                         \
   }
   YK_CASE(YK_F32, float, YK_F32, float)
@@ -375,4 +384,226 @@ extern "C" int yk_latent_attention(const float* q_lat, const void* pages, int dt
 #undef YK_RPL
 #undef YK_LAUNCH
   return yk_fail("latent_attention: unsupported dtype");
+}
+
+// ------------------------------------------------------------------ attention on the matrix cores
+// bfloat16 pages, rows of 32 KS elements of which the first 16 CT are the latent; beside the page
+// rows [slot][width] the latent is kept once more transposed, [column][slot], so that both products
+// take their first operand from memory as it lies there, 16 bytes a lane:
+//   S^T = K . Q^T   (first operand: 16 page rows x 32 elements; second: the queries, in registers)
+//   O^T = C^T . P^T (first operand: 16 latent columns x 32 slots of the transposed pages)
+// A wave owns 16 columns = (token, head) pairs of one tile: the heads of a token (16 at a time), or
+// several tokens' heads where a model has fewer than 16.  It walks the keys in groups of 32; within
+// a group the rows of the two score products are assigned to keys so that afterwards lane group g
+// holds the probabilities of keys 8g .. 8g + 7 in order (row i is key 8 (i / 4) + i % 4, + 4 for the
+// second product), which is the second operand of the other product as it stands.  Each lane keeps
+// its column's running maximum and sum.  The four waves of a workgroup take four tiles that follow
+// each other, so they ask for the same rows at about the same time.  With n_splits > 1 the groups of
+// keys are divided among gridDim.z workgroups, which leave unnormalised sums, maxima and sums of
+// weights for a merging kernel.
+typedef __bf16 lat_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float lat_f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t lat_u32x4_t __attribute__((ext_vector_type(4)));
+union LatFrag {
+  lat_u32x4_t u;
+  lat_bf16x8_t v;
+  bf16_t h[8];
+};
+
+template <int KS, int CT>
+__global__ __launch_bounds__(256, 1) void latent_attention_mfma_kernel(
+    const float* __restrict__ q_lat, const bf16_t* __restrict__ kpages, const bf16_t* __restrict__ vpages,
+    const int32_t* __restrict__ tiles, int n_tiles, const int32_t* __restrict__ block_table, int table_width, int page_size,
+    int n_heads, float scale_log2, int n_splits, float* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+  constexpr int WIDTH = 32 * KS, RANK = 16 * CT;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int tile_i = blockIdx.x * 4 + wave;
+  if (tile_i >= n_tiles) return;
+  const int r = lane % 16, g = lane / 16;
+  const int32_t* tile = tiles + 4 * tile_i;
+  const int seq = tile[0], tok0 = tile[1], count = tile[2], pos0 = tile[3];
+  const int chunk = blockIdx.y, split = blockIdx.z;
+  const int hpt = n_heads < 16 ? n_heads : 16;
+  const int tt = r / hpt, hh = r % hpt, head = chunk * 16 + hh;
+  const bool col_ok = tt < count && head < n_heads;
+  const int my_pos = pos0 + (col_ok ? tt : 0);
+  const int last = pos0 + count - 1;
+
+  LatFrag qf[KS];
+  {
+    const float* qp = q_lat + (static_cast<size_t>(tok0 + (col_ok ? tt : 0)) * n_heads + (col_ok ? head : 0)) * WIDTH + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const float4 a = *reinterpret_cast<const float4*>(qp + 32 * ks), b = *reinterpret_cast<const float4*>(qp + 32 * ks + 4);
+      qf[ks].u[0] = col_ok ? pack_bf16x2(a.x, a.y) : 0u;
+      qf[ks].u[1] = col_ok ? pack_bf16x2(a.z, a.w) : 0u;
+      qf[ks].u[2] = col_ok ? pack_bf16x2(b.x, b.y) : 0u;
+      qf[ks].u[3] = col_ok ? pack_bf16x2(b.z, b.w) : 0u;
+    }
+  }
+  const int groups = last / 32 + 1;
+  const int per = (groups + n_splits - 1) / n_splits;
+  const int g_lo = min(groups, split * per), g_hi = min(groups, g_lo + per);
+  const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
+
+  float m = -INFINITY, l = 0.f;
+  lat_f32x4_t acc[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) acc[ct] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int grp = g_lo; grp < g_hi; ++grp) {
+    const int k0 = grp * 32;
+    const size_t page = static_cast<size_t>(bt[k0 / page_size]);
+    const int slot0 = k0 % page_size;
+    lat_f32x4_t s[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      s[sb] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
+      // the page row behind row r of this product (rows that do not exist yet: the last one that does)
+      const int kl = min(8 * (r / 4) + 4 * sb + r % 4, last - k0);
+      const bf16_t* krow = kpages + (page * page_size + slot0 + kl) * WIDTH + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        LatFrag kf;
+        kf.u = *reinterpret_cast<const lat_u32x4_t*>(krow + 32 * ks);
+        s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks].v, s[sb], 0, 0, 0);
+      }
+    }
+    // this lane: column r, keys k0 + 8 g + 4 sb + j
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int key = k0 + 8 * g + 4 * sb + j;
+        s[sb][j] = key <= my_pos ? s[sb][j] * scale_log2 : -INFINITY;
+        tmax = fmaxf(tmax, s[sb][j]);
+      }
+    tmax = column_lanes_max(tmax);
+    const float m_new = fmaxf(m, tmax);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+    float psum = 0.f;
+    LatFrag pf;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s[sb][j] = __builtin_amdgcn_exp2f(s[sb][j] - m_safe);
+        psum += s[sb][j];
+      }
+      pf.u[2 * sb] = pack_bf16x2(s[sb][0], s[sb][1]);
+      pf.u[2 * sb + 1] = pack_bf16x2(s[sb][2], s[sb][3]);
+    }
+    l = l * alpha + psum;
+    m = m_new;
+    const bool ragged = k0 + 32 > last + 1;  // slots behind the last key hold whatever was there
+    const bf16_t* vcol = vpages + (page * RANK + r) * page_size + slot0 + 8 * g;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      LatFrag vf;
+      vf.u = *reinterpret_cast<const lat_u32x4_t*>(vcol + static_cast<size_t>(16 * ct) * page_size);
+      if (ragged) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (k0 + 8 * g + e > last) vf.h[e] = 0;
+      }
+      acc[ct] *= alpha;
+      acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[ct], 0, 0, 0);
+    }
+  }
+  l = column_lanes_sum(l);
+  // acc[ct][j]: latent column 16 ct + 4 g + j of this lane's column r
+  if (n_splits == 1) {
+    if (!col_ok) return;
+    const float inv = 1.f / l;
+    float* o = out + (static_cast<size_t>(tok0 + tt) * n_heads + head) * RANK + 4 * g;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+      *reinterpret_cast<float4*>(o + 16 * ct) = make_float4(acc[ct][0] * inv, acc[ct][1] * inv, acc[ct][2] * inv, acc[ct][3] * inv);
+    return;
+  }
+  const size_t part = (static_cast<size_t>(tile_i) * gridDim.y + chunk) * n_splits + split;
+  float* o = ws_o + (part * 16 + r) * RANK + 4 * g;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) *reinterpret_cast<float4*>(o + 16 * ct) = make_float4(acc[ct][0], acc[ct][1], acc[ct][2], acc[ct][3]);
+  if (g == 0) {
+    ws_ml[(part * 16 + r) * 2] = m;
+    ws_ml[(part * 16 + r) * 2 + 1] = l;
+  }
+}
+
+// one workgroup per (tile, head chunk): column r's splits merged with weights 2^(m_s - max m), in the order of s
+__global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                                                     const int32_t* __restrict__ tiles, int n_heads, int rank,
+                                                                     int n_splits, float* __restrict__ out) {
+  const int tile_i = blockIdx.x, chunk = blockIdx.y;
+  const int32_t* tile = tiles + 4 * tile_i;
+  const int tok0 = tile[1], count = tile[2];
+  const int hpt = n_heads < 16 ? n_heads : 16;
+  const size_t part0 = (static_cast<size_t>(tile_i) * gridDim.y + chunk) * n_splits;
+  for (int i = threadIdx.x; i < 16 * rank; i += blockDim.x) {
+    const int r = i / rank, c = i % rank;
+    const int tt = r / hpt, head = chunk * 16 + r % hpt;
+    if (tt >= count || head >= n_heads) continue;
+    float m_max = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, ws_ml[((part0 + s) * 16 + r) * 2]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float w = exp2f(ws_ml[((part0 + s) * 16 + r) * 2] - m_max);
+      num = fmaf(w, ws_o[((part0 + s) * 16 + r) * rank + c], num);
+      den = fmaf(w, ws_ml[((part0 + s) * 16 + r) * 2 + 1], den);
+    }
+    out[(static_cast<size_t>(tok0 + tt) * n_heads + head) * rank + c] = num / den;
+  }
+}
+
+// sizes the matrix-core form is built for: (page row, latent) = (576, 512), (320, 256), (160, 128), (96, 64)
+extern "C" int yk_latent_mfma_ok(int kv_rank, int rot_dim, int page_size) {
+  const int w = kv_rank + rot_dim;
+  const bool size_ok = (w == 576 && kv_rank == 512) || (w == 320 && kv_rank == 256) || (w == 160 && kv_rank == 128) ||
+                       (w == 96 && kv_rank == 64);
+  return size_ok && page_size % 32 == 0 ? 1 : 0;
+}
+
+extern "C" int yk_latent_mfma_tile_tokens(int n_heads) { return n_heads >= 16 ? 1 : 16 / n_heads; }
+
+// floats of workspace a launch with these tiles and splits needs
+extern "C" size_t yk_latent_mfma_workspace(int n_tiles, int n_heads, int kv_rank, int n_splits) {
+  if (n_splits <= 1) return 0;
+  const size_t parts = static_cast<size_t>(n_tiles) * ((n_heads + 15) / 16) * n_splits;
+  return parts * 16 * (kv_rank + 2);
+}
+
+extern "C" int yk_latent_attention_mfma(const float* q_lat, const void* kpages, const void* vpages, const int32_t* tiles,
+                                        int n_tiles, const int32_t* block_table, int table_width, int page_size, int n_heads,
+                                        int kv_rank, int rot_dim, float scale, int n_splits, float* workspace,
+                                        size_t workspace_floats, float* out, hipStream_t stream) {
+  YK_REQUIRE(yk_latent_mfma_ok(kv_rank, rot_dim, page_size), "latent_attention_mfma: sizes the matrix-core form is not built for");
+  YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && table_width > 0 && n_splits >= 1 && n_splits <= 256, "latent_attention_mfma: bad sizes");
+  YK_REQUIRE(workspace_floats >= yk_latent_mfma_workspace(n_tiles, n_heads, kv_rank, n_splits) && (n_splits == 1 || workspace != nullptr),
+             "latent_attention_mfma: the workspace is too small");
+  if (n_tiles == 0) return 0;
+  const int chunks = (n_heads + 15) / 16;
+  dim3 grid((n_tiles + 3) / 4, chunks, n_splits);
+  const float scale_log2 = scale * 1.4426950408889634f;
+  float* ws_o = workspace;
+  float* ws_ml = workspace == nullptr ? nullptr : workspace + static_cast<size_t>(n_tiles) * chunks * n_splits * 16 * kv_rank;
+#define YK_CASE(KS, CT)                                                                                                      \
+  if (kv_rank + rot_dim == 32 * KS && kv_rank == 16 * CT) {                                                                  \
+    latent_attention_mfma_kernel<KS, CT><<<grid, 256, 0, stream>>>(                                                          \
+        q_lat, static_cast<const bf16_t*>(kpages), static_cast<const bf16_t*>(vpages), tiles, n_tiles, block_table,          \
+        table_width, page_size, n_heads, scale_log2, n_splits, out, ws_o, ws_ml);                                            \
+    if (yk_check_launch("latent_attention_mfma") != 0) return -1;                                                            \
+  }
+  YK_CASE(18, 32)
+  YK_CASE(10, 16)
+  YK_CASE(5, 8)
+  YK_CASE(3, 4)
+#undef YK_CASE
+  if (n_splits > 1) {
+    latent_attention_merge_kernel<<<dim3(n_tiles, chunks), 256, 0, stream>>>(ws_o, ws_ml, tiles, n_heads, kv_rank, n_splits, out);
+    return yk_check_launch("latent_attention_merge");
+  }
+  return 0;
 }

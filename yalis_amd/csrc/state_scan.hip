@@ -7,9 +7,9 @@
 //
 // The columns of S never meet: column e needs k_t, q_t, a_t, beta_t and its own v_t[e] only.  So a
 // column lives in the registers of a group of TPC lanes (lane s of the group holds the rows s,
-// s + TPC, s + 2 TPC, ...; 16 rows a lane), the two sums over rows are exchanges inside the group,
-// and a workgroup walks a request's span token by token with k, q and the decays of the next few
-// tokens staged in LDS.  Decays, write strengths and unit norms are made here, in float32, from the
+// 16 s .. 16 s + 15), the two sums over rows are exchanges inside the group, and a workgroup walks a
+// request's span token by token with k, q and the decays of the next 32 tokens staged in LDS (a wave
+// per token and vector makes the unit norm while it stages), read back 16 bytes at a time.  Decays, write strengths and unit norms are made here, in float32, from the
 // projections' raw outputs:
 //   decay per head:     exp(-exp(A_log[h]) * softplus(x[n, h] + dt_bias[h]))
 //   decay per channel:  sigmoid(z[n, h, i] + bias[h, i]) ^ (1 / tau)  =  exp(logsigmoid(.) / tau)
@@ -24,54 +24,99 @@
 
 #include "common.h"
 
-constexpr int kScanRows = 16;    // rows of S a lane holds
-constexpr int kScanTokens = 16;  // tokens staged at a time
+constexpr int kScanRows = 16;    // rows of S a lane holds: sub * 16 .. sub * 16 + 15 of its column
+constexpr int kScanTokens = 32;  // tokens staged at a time (fewer where LDS would not hold them)
 
 __device__ __forceinline__ float scan_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 
-template <typename T>
+// the sum over the TPC lanes of a column (lanes that differ in their low bits)
+template <int TPC>
+__device__ __forceinline__ float column_sum(float v) {
+#pragma unroll
+  for (int o = TPC / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+// LDS per staged token: k and q padded to TPC * 16 floats each (rows past dim are zeros, so nobody
+// asks whether a row exists), the per-channel decays likewise where there are any
+template <typename T, int TPC>
 __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     const T* __restrict__ qkv, int qkv_stride, int n_heads, int n_kv, int dim, int vdim, float* __restrict__ state,
     const int32_t* __restrict__ seq_qstart, const int32_t* __restrict__ seq_qlen, const int32_t* __restrict__ state_slots,
     float q_scale, float unit_eps, int decay_mode, const float* __restrict__ decay, int decay_stride, int decay_col,
     const float* __restrict__ decay_p0, const float* __restrict__ decay_p1, float tau, const float* __restrict__ beta,
-    int beta_stride, int beta_col, int tpc, float* __restrict__ out) {
+    int beta_stride, int beta_col, int chunk, float* __restrict__ out) {
   extern __shared__ float lds[];
-  // [kScanTokens] x (k[dim], q[dim], a[dim or 1]), v[kScanTokens][cols], beta[kScanTokens], inv_k, inv_q
-  const int cols_per_block = blockDim.x / tpc;
-  float* ks = lds;
-  float* qs = ks + kScanTokens * dim;
-  float* as = qs + kScanTokens * dim;
-  const int a_w = decay_mode == 1 ? dim : 1;
-  float* vs = as + kScanTokens * a_w;
-  float* bs = vs + kScanTokens * cols_per_block;
-  float* inv = bs + kScanTokens;  // [kScanTokens][2]
+  constexpr int DP = TPC * kScanRows;  // padded key channels
+  const int cols_per_block = blockDim.x / TPC;
+  float* ks = lds;                                        // [chunk][DP]
+  float* qs = ks + chunk * DP;                            // [chunk][DP]
+  float* as = qs + chunk * DP;                            // [chunk][DP] (per channel) or [chunk]
+  float* vs = as + chunk * (decay_mode == 1 ? DP : 1);    // [chunk][cols_per_block]
+  float* bs = vs + chunk * cols_per_block;                // [chunk]
 
   const int seq = blockIdx.x, h = blockIdx.y, kvh = h / (n_heads / n_kv);
   const int col0 = blockIdx.z * cols_per_block;
-  const int sub = threadIdx.x % tpc, col_local = threadIdx.x / tpc, col = col0 + col_local;
+  const int sub = threadIdx.x % TPC, col_local = threadIdx.x / TPC, col = col0 + col_local;
   const bool has_col = col < vdim;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, n_waves = blockDim.x / kWave;
   const int q0 = seq_qstart[seq], ql = seq_qlen[seq];
   float* S_head = state + (static_cast<size_t>(state_slots[seq]) * n_heads + h) * dim * vdim;
+  const bool delta = beta != nullptr;
 
   float S[kScanRows];
 #pragma unroll
   for (int r = 0; r < kScanRows; ++r) {
-    const int i = r * tpc + sub;
+    const int i = sub * kScanRows + r;
     S[r] = has_col && i < dim ? S_head[static_cast<size_t>(i) * vdim + col] : 0.f;
   }
   const int kd = n_kv * dim;
-  for (int t0 = 0; t0 < ql; t0 += kScanTokens) {
-    const int nt = min(kScanTokens, ql - t0);
-    __syncthreads();
-    for (int i = threadIdx.x; i < nt * dim; i += blockDim.x) {
-      const int t = i / dim, c = i % dim;
-      const T* row = qkv + static_cast<size_t>(q0 + t0 + t) * qkv_stride;
-      qs[i] = to_f32<T>(row[kvh * dim + c]);
-      ks[i] = to_f32<T>(row[kd + kvh * dim + c]);
-      if (decay_mode == 1) {
-        const float z = decay[static_cast<size_t>(q0 + t0 + t) * decay_stride + decay_col + h * dim + c] + decay_p0[h * dim + c];
-        as[i] = expf(-scan_softplus(-z) / tau);  // sigmoid(z)^(1/tau)
+  for (int t0 = 0; t0 < ql; t0 += chunk) {
+    const int nt = min(chunk, ql - t0);
+    __syncthreads();  // the chunk before has been read
+    // q and k of the chunk's tokens to LDS, every load of a thread asked for before the first is used
+    // (one after the other they cost a round trip to memory each)
+    {
+      const float q_mul = unit_eps >= 0.f ? 1.f : q_scale;
+      const int total = 2 * nt * DP;
+      for (int i0 = threadIdx.x; i0 < total; i0 += 8 * blockDim.x) {
+        float x[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = i0 + j * blockDim.x;
+          const int item = i / DP, c = i % DP, t = item >> 1, is_k = item & 1;
+          x[j] = i < total && c < dim
+                     ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + (is_k ? kd : 0) + kvh * dim + c])
+                     : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = i0 + j * blockDim.x;
+          if (i < total) {
+            const int item = i / DP, c = i % DP, t = item >> 1, is_k = item & 1;
+            ((is_k ? ks : qs) + t * DP)[c] = is_k ? x[j] : x[j] * q_mul;
+          }
+        }
+      }
+    }
+    if (decay_mode == 1) {
+      const int total = nt * DP;
+      for (int i0 = threadIdx.x; i0 < total; i0 += 8 * blockDim.x) {
+        float z[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = i0 + j * blockDim.x;
+          const int t = i / DP, c = i % DP;
+          z[j] = i < total && c < dim
+                     ? decay[static_cast<size_t>(q0 + t0 + t) * decay_stride + decay_col + h * dim + c] + decay_p0[h * dim + c]
+                     : INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = i0 + j * blockDim.x;
+          // sigmoid(z)^(1/tau); channels past dim decay to nothing (their rows of S are zeros anyway)
+          if (i < total) as[i] = i % DP < dim ? expf(-scan_softplus(-z[j]) / tau) : 0.f;
+        }
       }
     }
     for (int i = threadIdx.x; i < nt * cols_per_block; i += blockDim.x) {
@@ -82,61 +127,70 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       const size_t n = static_cast<size_t>(q0 + t0 + t);
       if (decay_mode == 0)
         as[t] = expf(-expf(decay_p0[h]) * scan_softplus(decay[n * decay_stride + decay_col + h] + decay_p1[h]));
-      bs[t] = beta != nullptr ? 1.f / (1.f + expf(-beta[n * beta_stride + beta_col + h])) : 1.f;
+      bs[t] = delta ? 1.f / (1.f + expf(-beta[n * beta_stride + beta_col + h])) : 1.f;
     }
     __syncthreads();
     if (unit_eps >= 0.f) {
-      // a thread per (token, q or k): the sum of squares in the order of the elements
-      for (int i = threadIdx.x; i < 2 * nt; i += blockDim.x) {
-        const float* x = (i & 1 ? ks : qs) + (i >> 1) * dim;
+      // a wave per token and vector: the sum of squares over the wave, the row scaled where it lies
+      for (int item = wave; item < 2 * nt; item += n_waves) {
+        float* row = ((item & 1) ? ks : qs) + (item >> 1) * DP;
         float ss = 0.f;
-        for (int c = 0; c < dim; ++c) ss = fmaf(x[c], x[c], ss);
-        inv[i] = 1.f / sqrtf(ss + unit_eps);
+        for (int c = lane; c < DP; c += kWave) ss = fmaf(row[c], row[c], ss);
+        const float mul = ((item & 1) ? 1.f : q_scale) / sqrtf(wave_sum(ss) + unit_eps);
+        for (int c = lane; c < DP; c += kWave) row[c] *= mul;
       }
       __syncthreads();
-      for (int i = threadIdx.x; i < nt * dim; i += blockDim.x) {
-        const int t = i / dim;
-        qs[i] = qs[i] * inv[2 * t] * q_scale;
-        ks[i] *= inv[2 * t + 1];
-      }
-    } else {
-      for (int i = threadIdx.x; i < nt * dim; i += blockDim.x) qs[i] *= q_scale;
     }
-    __syncthreads();
     for (int t = 0; t < nt; ++t) {
-      const float* kt = ks + t * dim;
-      const float* qt = qs + t * dim;
-      const float* at = as + t * a_w;
+      const float4* kt = reinterpret_cast<const float4*>(ks + t * DP + sub * kScanRows);
+      const float4* qt = reinterpret_cast<const float4*>(qs + t * DP + sub * kScanRows);
       float kr[kScanRows];
-      float sk = 0.f;
 #pragma unroll
-      for (int r = 0; r < kScanRows; ++r) {
-        const int i = r * tpc + sub;
-        const bool in = i < dim;
-        kr[r] = in ? kt[i] : 0.f;
-        const float a = decay_mode == 1 ? (in ? at[i] : 0.f) : at[0];
-        S[r] *= a;
-        sk = fmaf(S[r], kr[r], sk);
+      for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
+        const float4 k4 = kt[r4];
+        kr[4 * r4] = k4.x; kr[4 * r4 + 1] = k4.y; kr[4 * r4 + 2] = k4.z; kr[4 * r4 + 3] = k4.w;
+      }
+      if (decay_mode == 1) {
+        const float4* at = reinterpret_cast<const float4*>(as + t * DP + sub * kScanRows);
+#pragma unroll
+        for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
+          const float4 a4 = at[r4];
+          S[4 * r4] *= a4.x; S[4 * r4 + 1] *= a4.y; S[4 * r4 + 2] *= a4.z; S[4 * r4 + 3] *= a4.w;
+        }
+      } else {
+        const float a = as[t];
+#pragma unroll
+        for (int r = 0; r < kScanRows; ++r) S[r] *= a;
       }
       float u = vs[t * cols_per_block + col_local];
-      if (beta != nullptr) {
-        for (int o = tpc / 2; o > 0; o >>= 1) sk += __shfl_xor(sk, o, kWave);
+      if (delta) {
+        // S^T k in four partial sums (rows r, r + 4, ...), then over the column's lanes
+        float p[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int r = 0; r < kScanRows; ++r) p[r % 4] = fmaf(S[r], kr[r], p[r % 4]);
+        const float sk = column_sum<TPC>((p[0] + p[1]) + (p[2] + p[3]));
         u = bs[t] * (u - sk);
       }
-      float so = 0.f;
+      float p[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int r = 0; r < kScanRows; ++r) {
-        const int i = r * tpc + sub;
-        S[r] = fmaf(kr[r], u, S[r]);
-        so = fmaf(S[r], i < dim ? qt[i] : 0.f, so);
+      for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
+        const float4 q4 = qt[r4];
+        S[4 * r4] = fmaf(kr[4 * r4], u, S[4 * r4]);
+        S[4 * r4 + 1] = fmaf(kr[4 * r4 + 1], u, S[4 * r4 + 1]);
+        S[4 * r4 + 2] = fmaf(kr[4 * r4 + 2], u, S[4 * r4 + 2]);
+        S[4 * r4 + 3] = fmaf(kr[4 * r4 + 3], u, S[4 * r4 + 3]);
+        p[0] = fmaf(S[4 * r4], q4.x, p[0]);
+        p[1] = fmaf(S[4 * r4 + 1], q4.y, p[1]);
+        p[2] = fmaf(S[4 * r4 + 2], q4.z, p[2]);
+        p[3] = fmaf(S[4 * r4 + 3], q4.w, p[3]);
       }
-      for (int o = tpc / 2; o > 0; o >>= 1) so += __shfl_xor(so, o, kWave);
+      const float so = column_sum<TPC>((p[0] + p[1]) + (p[2] + p[3]));
       if (has_col && sub == 0) out[(static_cast<size_t>(q0 + t0 + t) * n_heads + h) * vdim + col] = so;
     }
   }
 #pragma unroll
   for (int r = 0; r < kScanRows; ++r) {
-    const int i = r * tpc + sub;
+    const int i = sub * kScanRows + r;
     if (has_col && i < dim) S_head[static_cast<size_t>(i) * vdim + col] = S[r];
   }
 }
@@ -162,21 +216,41 @@ extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, 
   while (tpc * kScanRows < dim) tpc *= 2;
   int threads = vdim * tpc;
   threads = std::min(256, (threads + kWave - 1) / kWave * kWave);
+  // (a decay per channel stages three padded rows a token: fewer threads where LDS would not hold more columns)
   const int cols = threads / tpc;
   dim3 grid(n_seqs, n_heads, (vdim + cols - 1) / cols);
-  const size_t lds = sizeof(float) * (static_cast<size_t>(kScanTokens) * (2 * dim + (decay_mode == 1 ? dim : 1) + cols + 3));
-  YK_REQUIRE(lds <= 64 * 1024, "linear_state_scan: the staged tokens do not fit in LDS");
-  if (dtype == YK_F32)
-    linear_state_scan_kernel<float><<<grid, threads, lds, stream>>>(
-        static_cast<const float*>(qkv), qkv_stride, n_heads, n_kv, dim, vdim, state, seq_qstart, seq_qlen, state_slots, q_scale,
-        unit_eps, decay_mode, decay, decay_stride, decay_col, decay_p0, decay_p1, tau, beta, beta_stride, beta_col, tpc, out);
-  else if (dtype == YK_BF16)
-    linear_state_scan_kernel<bf16_t><<<grid, threads, lds, stream>>>(
-        static_cast<const bf16_t*>(qkv), qkv_stride, n_heads, n_kv, dim, vdim, state, seq_qstart, seq_qlen, state_slots, q_scale,
-        unit_eps, decay_mode, decay, decay_stride, decay_col, decay_p0, decay_p1, tau, beta, beta_stride, beta_col, tpc, out);
-  else
-    return yk_fail("linear_state_scan: unsupported dtype");
-  return yk_check_launch("linear_state_scan");
+  const size_t dp = static_cast<size_t>(tpc) * kScanRows;
+  int chunk = kScanTokens;
+  const size_t per_token = sizeof(float) * (2 * dp + (decay_mode == 1 ? dp : 1) + cols + 1);
+  while (chunk > 4 && chunk * per_token > 100 * 1024) chunk /= 2;
+  const size_t lds = chunk * per_token;
+  YK_REQUIRE(lds <= 128 * 1024, "linear_state_scan: the staged tokens do not fit in LDS");
+#define YK_LAUNCH(T, TPC)                                                                                                       \
+  {                                                                                                                             \
+    auto kern = linear_state_scan_kernel<T, TPC>;                                                                               \
+    if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                               static_cast<int>(lds)) != hipSuccess)                                            \
+      return yk_fail("linear_state_scan: the staged tokens do not fit in LDS");                                                 \
+    kern<<<grid, threads, lds, stream>>>(static_cast<const T*>(qkv), qkv_stride, n_heads, n_kv, dim, vdim, state, seq_qstart,   \
+                                         seq_qlen, state_slots, q_scale, unit_eps, decay_mode, decay, decay_stride, decay_col,  \
+                                         decay_p0, decay_p1, tau, beta, beta_stride, beta_col, chunk, out);                     \
+    return yk_check_launch("linear_state_scan");                                                                                \
+  }
+#define YK_TPC(T)                   \
+  switch (tpc) {                    \
+    case 1: YK_LAUNCH(T, 1)         \
+    case 2: YK_LAUNCH(T, 2)         \
+    case 4: YK_LAUNCH(T, 4)         \
+    case 8: YK_LAUNCH(T, 8)         \
+    case 16: YK_LAUNCH(T, 16)       \
+    case 32: YK_LAUNCH(T, 32)       \
+    default: YK_LAUNCH(T, 64)       \
+  }
+  if (dtype == YK_F32) YK_TPC(float)
+  if (dtype == YK_BF16) YK_TPC(bf16_t)
+#undef YK_TPC
+#undef YK_LAUNCH
+  return yk_fail("linear_state_scan: unsupported dtype");
 }
 
 // --------------------------------------------------------------- the read-out's norm and gate

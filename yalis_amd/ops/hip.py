@@ -90,7 +90,14 @@ _SIGNATURES = {
     "yk_scale_rows": ([_vp, _c_float, _c_size_t, _vp], _c_int),
     "yk_latent_prepare": (
         [_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _vp, _vp,
-         _c_int, _vp],
+         _c_int, _vp, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_latent_mfma_ok": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_latent_mfma_tile_tokens": ([_c_int], _c_int),
+    "yk_latent_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int], _c_size_t),
+    "yk_latent_attention_mfma": (
+        [_vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_size_t, _vp, _vp],
         _c_int,
     ),
     "yk_head_linear": (
@@ -1334,11 +1341,12 @@ class HipOps:
 
     # ------------------------------------------------------------- attention over one latent per token
     def latent_prepare(self, proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, rot_dim=0, kv_norm=None, rotation=None,
-                       positions=None, pages=None, slots=None, page_size=0) -> torch.Tensor:
+                       positions=None, pages=None, slots=None, page_size=0, values=None) -> torch.Tensor:
         """From the stacked down-projection's rows ``proj`` [N, >= q_rank (+ sections)]: the query
         latent rmsnorm(proj[:, :q_rank]) * q_norm [N, q_rank]; and, with ``kv_rank`` > 0, each token's
         page row [rmsnorm(proj[:, kv_col : kv_col + kv_rank]) * kv_norm | the next rot_dim elements turned
-        by the token's position] written at its slot of ``pages`` [pages, 1, page_size, kv_rank + rot_dim]."""
+        by the token's position] written at its slot of ``pages`` [pages, 1, page_size, kv_rank + rot_dim], and
+        the normed latent once more, transposed, into ``values`` [pages, 1, kv_rank, page_size] where given."""
         self._rows(proj, "latent_prepare input")
         n = proj.shape[0]
         if proj.dtype != act_dtype:
@@ -1354,6 +1362,9 @@ class HipOps:
             if pages is None or pages.dtype != act_dtype or not pages.is_contiguous() or pages.dim() != 4 or pages.shape[1] != 1 \
                     or pages.shape[2] != page_size or pages.shape[3] != kv_rank + rot_dim:
                 raise KernelError(f"latent_prepare: pages {None if pages is None else tuple(pages.shape)} do not hold rows of {kv_rank + rot_dim}")
+            if values is not None and (values.dtype != act_dtype or not values.is_contiguous()
+                                       or tuple(values.shape) != (pages.shape[0], 1, kv_rank, page_size)):
+                raise KernelError(f"latent_prepare: transposed pages {tuple(values.shape)} do not match the pages")
             if rot_dim:
                 if rotation is None or rotation.rotary_dim != rot_dim:
                     raise KernelError("latent_prepare: the rotation must cover the rotated part exactly")
@@ -1361,7 +1372,8 @@ class HipOps:
         self._check(self.lib.yk_latent_prepare(
             proj.data_ptr(), proj.stride(0), _code(proj.dtype), q_rank, q_norm.data_ptr(), _code(q_norm.dtype), float(eps),
             c_q.data_ptr(), kv_col, kv_rank, rot_dim, _ptr(kv_norm), _ptr(positions), _ptr(cos), _ptr(sin), inter, max_pos,
-            _ptr(pages) if kv_rank else None, _ptr(slots) if kv_rank else None, n, self._stream()))
+            _ptr(pages) if kv_rank else None, _ptr(values) if kv_rank else None, page_size, _ptr(slots) if kv_rank else None, n,
+            self._stream()))
         return c_q
 
     def head_linear(self, x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0):
@@ -1397,11 +1409,24 @@ class HipOps:
             n, self._stream()))
         return out
 
-    def latent_tile_tokens(self, n_heads: int) -> int:
-        """Consecutive tokens of a request that one workgroup of ``latent_attention`` takes."""
-        return self._ask("yk_latent_tile_tokens", n_heads)
+    def latent_attention_on_matrix_cores(self, act_dtype: torch.dtype, kv_rank: int, rot_dim: int, page_size: int) -> bool:
+        """Whether ``latent_attention`` has its matrix-core form for these sizes; that form reads the
+        latent a second time from transposed pages (``values``), which the caller then has to keep."""
+        return act_dtype == torch.bfloat16 and bool(self._ask("yk_latent_mfma_ok", kv_rank, rot_dim, page_size))
 
-    def latent_attention(self, q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None) -> torch.Tensor:
+    def latent_tile_tokens(self, n_heads: int, matrix_cores: bool = False) -> int:
+        """Consecutive tokens of a request that one tile of ``latent_attention`` takes."""
+        return self._ask("yk_latent_mfma_tile_tokens" if matrix_cores else "yk_latent_tile_tokens", n_heads)
+
+    @staticmethod
+    def latent_attention_splits(n_tiles: int, n_heads: int, max_ctx: int) -> int:
+        """Into how many workgroups the matrix-core form divides the keys of a tile: none while the
+        tiles alone make some hundreds of waves; else as many as that takes, each with at least 128 keys."""
+        waves = n_tiles * -(-n_heads // 16)
+        return max(1, min(-(-512 // max(waves, 1)), max(1, -(-max_ctx // 32) // 4), 64))
+
+    def latent_attention(self, q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None, values=None,
+                         splits: Optional[int] = None) -> torch.Tensor:
         """Causal softmax attention of ``q_lat`` (float32 [N, heads * (kv_rank + rot_dim)]) over the page
         rows [c | kr] of each token's request: scores q . row * scale, the result sum_j p_j c_j as
         float32 [N, heads * kv_rank].  ``tiles``: the step's spans cut into ``latent_tile_tokens`` tokens
@@ -1416,6 +1441,20 @@ class HipOps:
             tiles = ctx.arrays[f"latent_tiles_{self.latent_tile_tokens(n_heads)}"]
         bt = ctx.arrays[f"block_table_g{group}"]
         out = torch.empty((n, n_heads * kv_rank), dtype=torch.float32, device=q_lat.device)
+        if values is not None:
+            # the matrix-core form: ``tiles`` are cut for it (latent_tile_tokens(heads, True))
+            if tiles is None or not self.latent_attention_on_matrix_cores(pages.dtype, kv_rank, rot_dim, page_size) or not values.is_contiguous() \
+                    or values.dtype != pages.dtype or tuple(values.shape) != (pages.shape[0], 1, kv_rank, page_size):
+                raise KernelError("latent_attention: transposed pages are for the matrix-core form, with tiles cut for it")
+            if splits is None:  # (given: tests and measurements force a number)
+                splits = self.latent_attention_splits(tiles.shape[0], n_heads, int(ctx.max_ctx))
+            floats = self.lib.yk_latent_mfma_workspace(tiles.shape[0], n_heads, kv_rank, splits)
+            ws = self._ws(floats) if floats else None
+            self._check(self.lib.yk_latent_attention_mfma(
+                q_lat.data_ptr(), pages.data_ptr(), values.data_ptr(), tiles.data_ptr(), tiles.shape[0], bt.data_ptr(), bt.shape[1],
+                page_size, n_heads, kv_rank, rot_dim, float(scale), splits, _ptr(ws), 0 if ws is None else ws.numel(), out.data_ptr(),
+                self._stream()))
+            return out
         self._check(self.lib.yk_latent_attention(
             q_lat.data_ptr(), pages.data_ptr(), _code(pages.dtype), tiles.data_ptr(), tiles.shape[0], bt.data_ptr(), bt.shape[1],
             page_size, n_heads, kv_rank, rot_dim, float(scale), out.data_ptr(), self._stream()))

@@ -7,7 +7,8 @@ key elements, value_dim value elements):
     k_head = W_uk,head c                  v_head = W_uv,head c
     score(i, j) = (q_i[:dim] . k_head,j + turn(q_i[dim:], i) . kr_j) * scale,  softmax over j <= i
     out = W_o concat_heads(sigmoid(W_g h)_head * sum_j p_ij v_head,j)
-A token's page row holds [c | kr] and nothing else; a layer may read another layer's pages
+A token's page row holds [c | kr] and nothing else (where the kernel library's matrix-core attention
+takes the sizes, c is kept a second time transposed, as value pages); a layer may read another layer's pages
 (``RunEntry.cache_from``) with W_uk, W_uv and queries of its own.
 
 The up-projections never touch the cached rows: since q[:dim] . (W_uk c) = (W_uk^T q[:dim]) . c and
@@ -74,8 +75,11 @@ class LatentAttention(Mixer):
         self.gate_col = self.kv_col + (up8(self.kv_rank + self.rot_dim) if self.projects_kv else 0)
         self.down_rows = self.gate_col + (self.n_heads if self.gate_name else 0)
         self.down_rows += -self.down_rows % 16
-        # consecutive tokens of a request that one workgroup of the attention takes
-        self.tile_tokens = int(rt.ops.latent_tile_tokens(self.n_heads))
+        # where the kernel library has its matrix-core attention for these sizes the latent is kept a second
+        # time, transposed, in value pages (that form's second product reads a column's slots side by side)
+        self.on_matrix_cores = bool(rt.ops.latent_attention_on_matrix_cores(rt.act_dtype, self.kv_rank, self.rot_dim, rt.page_size))
+        # consecutive tokens of a request that one tile of the attention takes
+        self.tile_tokens = int(rt.ops.latent_tile_tokens(self.n_heads, self.on_matrix_cores))
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         n, H = self.names, self.n_heads
@@ -114,7 +118,7 @@ class LatentAttention(Mixer):
 
     def kv_need(self) -> KVNeed:
         # one row of kv_rank + rot_dim elements per token and no values: the row serves as both
-        return KVNeed(1, self.kv_rank + self.rot_dim, None, 0)
+        return KVNeed(1, self.kv_rank + self.rot_dim, None, self.kv_rank if self.on_matrix_cores else 0)
 
     def products(self):
         H = self.n_heads
@@ -122,25 +126,26 @@ class LatentAttention(Mixer):
 
     def step_inputs(self):
         n = self.tile_tokens
-        return {f"latent_tiles_{n}": lambda hb: attention_tiles(hb, n)}
+        # (the tiles with the most keys first: their workgroups start first, the short ones fill the end)
+        return {f"latent_tiles_{n}": lambda hb: attention_tiles(hb, n, longest_first=True)}
 
     def forward(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
         ops, act = self.rt.ops, self.rt.act_dtype
         if site.owns_cache != self.projects_kv:
             raise RuntimeError(f"{self.prefix}: a layer whose run entries both own and borrow caches is not offered")
         proj = ops.linear(h, self.w_down, act)
-        pages, _ = site.kv()
+        pages, values = site.kv()
         c_q = ops.latent_prepare(
             proj, self.q_rank, self.w_qn, self.eps, act, kv_col=self.kv_col, kv_rank=self.kv_rank if site.owns_cache else 0,
             rot_dim=self.rot_dim, kv_norm=self.w_kvn, rotation=self.rotation, positions=ctx.arrays["positions"], pages=pages,
-            slots=ctx.arrays[f"slots_g{site.group}"], page_size=self.rt.page_size,
+            slots=ctx.arrays[f"slots_g{site.group}"], page_size=self.rt.page_size, values=values,
         )
         q = ops.linear(c_q, self.w_uq, act)
         # queries in the latent's space: [W_uk^T q[:dim] | q[dim:] turned by the position], float32
         q_lat = ops.head_linear(q, self.w_uk, self.n_heads, self.head_dim, self.kv_rank, torch.float32, tail=self.rot_dim,
                                 rotation=self.rotation, positions=ctx.arrays["positions"])
         o_lat = ops.latent_attention(q_lat, pages, self.n_heads, self.kv_rank, self.rot_dim, self.scale, ctx, site.group,
-                                     self.rt.page_size, tiles=ctx.arrays[f"latent_tiles_{self.tile_tokens}"])
+                                     self.rt.page_size, tiles=ctx.arrays[f"latent_tiles_{self.tile_tokens}"], values=values)
         o = ops.head_linear(o_lat, self.w_uv_t, self.n_heads, self.kv_rank, self.value_dim, act,
                             gate=proj if self.gate_name else None, gate_col=self.gate_col)
         return ops.linear(o, self.w_o, act, partial_ok=True)
