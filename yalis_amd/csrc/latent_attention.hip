@@ -96,18 +96,25 @@ extern "C" int yk_latent_prepare(const void* proj, int proj_stride, int dtype, i
 }
 
 // ------------------------------------------------------------------------- per-head products
-constexpr int kHeadTokens = 8;  // tokens a workgroup multiplies by one head's matrix
+constexpr int kHeadTokens = 8;   // tokens a workgroup multiplies by one head's matrix
+constexpr int kHeadOut = 64;     // output columns a workgroup makes
+// SLICES groups of 64 threads divide the input elements among them: four for a handful of tokens (more
+// waves on a product that is all latency), one for many (no meeting in LDS, every weight read once a tile)
 
-template <typename TX, typename TW, typename TO>
-__global__ __launch_bounds__(256) void head_linear_kernel(
+// out[n, h, o] = sum_i x[n, h, i] w[h][i][o] for a tile of kHeadTokens tokens, one head and kHeadOut
+// columns; thread (slice, column) sums every fourth input element, the slices meet in LDS.  TX: the
+// input's and TG the gate's element type.
+template <typename TX, typename TW, typename TG, typename TO, int kHeadSlices>
+__global__ __launch_bounds__(kHeadOut * kHeadSlices) void head_linear_kernel(
     const TX* __restrict__ x, int x_stride, const TW* __restrict__ w, TO* __restrict__ out, int out_stride, int in_dim,
     int out_dim, int tail, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
-    const float* __restrict__ sin_t, int interleaved, const TX* __restrict__ gate, int gate_stride, int gate_col,
+    const float* __restrict__ sin_t, int interleaved, const TG* __restrict__ gate, int gate_stride, int gate_col,
     int n_tokens) {
-  extern __shared__ float xs[];  // [kHeadTokens][in_dim + tail]
-  const int n0 = blockIdx.x * kHeadTokens, h = blockIdx.y;
+  extern __shared__ float xs[];  // [kHeadTokens][in_dim + tail], then [kHeadSlices][kHeadTokens][kHeadOut]
+  const int n0 = blockIdx.x * kHeadTokens, h = blockIdx.y, o0 = blockIdx.z * kHeadOut;
   const int count = min(kHeadTokens, n_tokens - n0);
   const int xw = in_dim + tail;
+  float* part = xs + kHeadTokens * xw;
   for (int i = threadIdx.x; i < kHeadTokens * xw; i += blockDim.x) {
     const int t = i / xw, c = i % xw;
     xs[i] = t < count ? to_f32<TX>(x[static_cast<size_t>(n0 + t) * x_stride + h * xw + c]) : 0.f;
@@ -115,21 +122,39 @@ __global__ __launch_bounds__(256) void head_linear_kernel(
   __syncthreads();
   const TW* wh = w + static_cast<size_t>(h) * in_dim * out_dim;
   const int ow = out_dim + tail;
-  for (int o = threadIdx.x; o < out_dim; o += blockDim.x) {
-    float acc[kHeadTokens];
+  const int slice = threadIdx.x / kHeadOut, o = o0 + threadIdx.x % kHeadOut;
+  float acc[kHeadTokens];
 #pragma unroll
-    for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
-    for (int i = 0; i < in_dim; ++i) {
-      const float wv = to_f32<TW>(wh[static_cast<size_t>(i) * out_dim + o]);
+  for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
+  if (o < out_dim) {
+    for (int i0 = slice; i0 < in_dim; i0 += 4 * kHeadSlices) {
+      float wv[4];
 #pragma unroll
-      for (int t = 0; t < kHeadTokens; ++t) acc[t] = fmaf(xs[t * xw + i], wv, acc[t]);
-    }
-    for (int t = 0; t < count; ++t) {
-      float v = acc[t];
-      if (gate != nullptr) v *= 1.f / (1.f + expf(-to_f32<TX>(gate[static_cast<size_t>(n0 + t) * gate_stride + gate_col + h])));
-      out[static_cast<size_t>(n0 + t) * out_stride + h * ow + o] = from_f32<TO>(v);
+      for (int j = 0; j < 4; ++j) {
+        const int i = i0 + j * kHeadSlices;
+        wv[j] = i < in_dim ? to_f32<TW>(wh[static_cast<size_t>(i) * out_dim + o]) : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = min(i0 + j * kHeadSlices, in_dim - 1);
+#pragma unroll
+        for (int t = 0; t < kHeadTokens; ++t) acc[t] = fmaf(xs[t * xw + i], wv[j], acc[t]);
+      }
     }
   }
+#pragma unroll
+  for (int t = 0; t < kHeadTokens; ++t) part[(slice * kHeadTokens + t) * kHeadOut + threadIdx.x % kHeadOut] = acc[t];
+  __syncthreads();
+  for (int i = threadIdx.x; i < count * kHeadOut; i += blockDim.x) {
+    const int t = i / kHeadOut, oc = i % kHeadOut;
+    if (o0 + oc >= out_dim) continue;
+    float v = 0.f;
+#pragma unroll
+    for (int sl = 0; sl < kHeadSlices; ++sl) v += part[(sl * kHeadTokens + t) * kHeadOut + oc];
+    if (gate != nullptr) v *= 1.f / (1.f + expf(-to_f32<TG>(gate[static_cast<size_t>(n0 + t) * gate_stride + gate_col + h])));
+    out[static_cast<size_t>(n0 + t) * out_stride + h * ow + o0 + oc] = from_f32<TO>(v);
+  }
+  if (blockIdx.z != 0) return;
   const int half = tail / 2;
   for (int i = threadIdx.x; i < count * half; i += blockDim.x) {
     const int t = i / half, j = i % half;
@@ -143,89 +168,43 @@ __global__ __launch_bounds__(256) void head_linear_kernel(
   }
 }
 
+// x, w, gate and out each float32 or bfloat16 (the gate in the output's dtype where the input is float32:
+// the way out of the latent; else in the input's)
 extern "C" int yk_head_linear(const void* x, int x_stride, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,
                               int n_heads, int in_dim, int out_dim, int tail, const int32_t* positions, const float* cos_t,
-                              const float* sin_t, int interleaved, const void* gate, int gate_stride, int gate_col,
-                              int n_tokens, hipStream_t stream) {
+                              const float* sin_t, int interleaved, const void* gate, int gate_dtype, int gate_stride,
+                              int gate_col, int n_tokens, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && in_dim > 0 && out_dim > 0 && tail >= 0 && tail % 2 == 0, "head_linear: bad sizes");
   YK_REQUIRE(x_stride >= n_heads * (in_dim + tail), "head_linear: the input's rows are shorter than its heads");
   YK_REQUIRE(tail == 0 || (positions != nullptr && cos_t != nullptr && sin_t != nullptr), "head_linear: a turned tail needs positions and tables");
-  const size_t lds = static_cast<size_t>(kHeadTokens) * (in_dim + tail) * sizeof(float);
-  YK_REQUIRE(lds <= 64 * 1024, "head_linear: heads of more than 2,048 input elements do not fit");
+  const int slices = n_tokens > 4 * kHeadTokens ? 1 : 4;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(kHeadTokens) * (in_dim + tail) + slices * kHeadTokens * kHeadOut);
+  YK_REQUIRE(lds <= 64 * 1024, "head_linear: heads of more than 1,700 input elements do not fit");
   if (n_tokens == 0) return 0;
-  dim3 grid((n_tokens + kHeadTokens - 1) / kHeadTokens, n_heads);
-  const int block = out_dim <= 64 ? 64 : out_dim <= 128 ? 128 : 256;
+  dim3 grid((n_tokens + kHeadTokens - 1) / kHeadTokens, n_heads, (out_dim + kHeadOut - 1) / kHeadOut);
   const int out_stride = n_heads * (out_dim + tail);
-#define YK_CASE(XD, TX, WD, TW, OD, TO)                                                                              \
-  if (x_dtype == XD && w_dtype == WD && out_dtype == OD) {                                                           \
-    head_linear_kernel<TX, TW, TO><<<grid, block, lds, stream>>>(                                                    \
-        static_cast<const TX*>(x), x_stride, static_cast<const TW*>(w), static_cast<TO*>(out), out_stride, in_dim,   \
-        out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TX*>(gate), gate_stride, gate_col,    \
-        n_tokens);                                                                                                   \
+  if (gate == nullptr) gate_dtype = out_dtype;
+#define YK_CASE(XD, TX, WD, TW, GD, TG, OD, TO)                                                                      \
+  if (x_dtype == XD && w_dtype == WD && gate_dtype == GD && out_dtype == OD) {                                       \
+    if (slices == 1)                                                                                                 \
+      head_linear_kernel<TX, TW, TG, TO, 1><<<grid, kHeadOut, lds, stream>>>(                                        \
+          static_cast<const TX*>(x), x_stride, static_cast<const TW*>(w), static_cast<TO*>(out), out_stride, in_dim, \
+          out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TG*>(gate), gate_stride, gate_col,  \
+          n_tokens);                                                                                                 \
+    else                                                                                                             \
+      head_linear_kernel<TX, TW, TG, TO, 4><<<grid, kHeadOut * 4, lds, stream>>>(                                    \
+          static_cast<const TX*>(x), x_stride, static_cast<const TW*>(w), static_cast<TO*>(out), out_stride, in_dim, \
+          out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TG*>(gate), gate_stride, gate_col,  \
+          n_tokens);                                                                                                 \
     return yk_check_launch("head_linear");                                                                           \
   }
-  YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
-  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_F32, float)
-  YK_CASE(YK_BF16, bf16_t, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_F32, float, YK_F32, float, YK_BF16, bf16_t, YK_BF16, bf16_t)
 #undef YK_CASE
   return yk_fail("head_linear: unsupported dtype combination");
-}
-
-// float32 rows in (the attention's sums over the latent), the activation dtype out, the gate in the
-// activation dtype: the same arithmetic with the gate's own element type
-template <typename TW, typename TG, typename TO>
-__global__ __launch_bounds__(256) void head_linear_out_kernel(
-    const float* __restrict__ x, int x_stride, const TW* __restrict__ w, TO* __restrict__ out, int out_stride, int in_dim,
-    int out_dim, const TG* __restrict__ gate, int gate_stride, int gate_col, int n_tokens) {
-  extern __shared__ float xs[];  // [kHeadTokens][in_dim]
-  const int n0 = blockIdx.x * kHeadTokens, h = blockIdx.y;
-  const int count = min(kHeadTokens, n_tokens - n0);
-  for (int i = threadIdx.x; i < kHeadTokens * in_dim; i += blockDim.x) {
-    const int t = i / in_dim, c = i % in_dim;
-    xs[i] = t < count ? x[static_cast<size_t>(n0 + t) * x_stride + h * in_dim + c] : 0.f;
-  }
-  __syncthreads();
-  const TW* wh = w + static_cast<size_t>(h) * in_dim * out_dim;
-  for (int o = threadIdx.x; o < out_dim; o += blockDim.x) {
-    float acc[kHeadTokens];
-#pragma unroll
-    for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
-    for (int i = 0; i < in_dim; ++i) {
-      const float wv = to_f32<TW>(wh[static_cast<size_t>(i) * out_dim + o]);
-#pragma unroll
-      for (int t = 0; t < kHeadTokens; ++t) acc[t] = fmaf(xs[t * in_dim + i], wv, acc[t]);
-    }
-    for (int t = 0; t < count; ++t) {
-      float v = acc[t];
-      if (gate != nullptr) v *= 1.f / (1.f + expf(-to_f32<TG>(gate[static_cast<size_t>(n0 + t) * gate_stride + gate_col + h])));
-      out[static_cast<size_t>(n0 + t) * out_stride + h * out_dim + o] = from_f32<TO>(v);
-    }
-  }
-}
-
-extern "C" int yk_head_linear_out(const float* x, int x_stride, const void* w, int w_dtype, void* out, int out_dtype,
-                                  int n_heads, int in_dim, int out_dim, const void* gate, int gate_stride, int gate_col,
-                                  int n_tokens, hipStream_t stream) {
-  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && in_dim > 0 && out_dim > 0, "head_linear_out: bad sizes");
-  YK_REQUIRE(x_stride >= n_heads * in_dim, "head_linear_out: the input's rows are shorter than its heads");
-  const size_t lds = static_cast<size_t>(kHeadTokens) * in_dim * sizeof(float);
-  YK_REQUIRE(lds <= 64 * 1024, "head_linear_out: heads of more than 2,048 input elements do not fit");
-  if (n_tokens == 0) return 0;
-  dim3 grid((n_tokens + kHeadTokens - 1) / kHeadTokens, n_heads);
-  const int block = out_dim <= 64 ? 64 : out_dim <= 128 ? 128 : 256;
-#define YK_CASE(WD, TW, OD, TO)                                                                                          \
-  if (w_dtype == WD && out_dtype == OD) {                                                                                \
-    head_linear_out_kernel<TW, TO, TO><<<grid, block, lds, stream>>>(x, x_stride, static_cast<const TW*>(w),             \
-                                                                     static_cast<TO*>(out), n_heads * out_dim, in_dim,   \
-                                                                     out_dim, static_cast<const TO*>(gate), gate_stride, \
-                                                                     gate_col, n_tokens);                                \
-    return yk_check_launch("head_linear_out");                                                                           \
-  }
-  YK_CASE(YK_F32, float, YK_F32, float)
-  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
-  YK_CASE(YK_F32, float, YK_BF16, bf16_t)
-#undef YK_CASE
-  return yk_fail("head_linear_out: unsupported dtype combination");
 }
 
 // --------------------------------------------------------------------------------- attention
@@ -533,28 +512,52 @@ __global__ __launch_bounds__(256, 1) void latent_attention_mfma_kernel(
   }
 }
 
-// one workgroup per (tile, head chunk): column r's splits merged with weights 2^(m_s - max m), in the order of s
-__global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+// one workgroup per (tile, head chunk, column): the column's splits merged with weights 2^(m_s - max m), in
+// the order of s; the weights are made once, by the first threads, and every thread's loads of a latent
+// column's parts are asked for together
+__global__ __launch_bounds__(128) void latent_attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                                      const int32_t* __restrict__ tiles, int n_heads, int rank,
                                                                      int n_splits, float* __restrict__ out) {
-  const int tile_i = blockIdx.x, chunk = blockIdx.y;
+  __shared__ float w[256];
+  __shared__ float inv_den;
+  const int tile_i = blockIdx.x, chunk = blockIdx.y, r = blockIdx.z;
   const int32_t* tile = tiles + 4 * tile_i;
   const int tok0 = tile[1], count = tile[2];
   const int hpt = n_heads < 16 ? n_heads : 16;
+  const int tt = r / hpt, head = chunk * 16 + r % hpt;
+  if (tt >= count || head >= n_heads) return;
   const size_t part0 = (static_cast<size_t>(tile_i) * gridDim.y + chunk) * n_splits;
-  for (int i = threadIdx.x; i < 16 * rank; i += blockDim.x) {
-    const int r = i / rank, c = i % rank;
-    const int tt = r / hpt, head = chunk * 16 + r % hpt;
-    if (tt >= count || head >= n_heads) continue;
+  if (threadIdx.x < kWave) {
     float m_max = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, ws_ml[((part0 + s) * 16 + r) * 2]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float w = exp2f(ws_ml[((part0 + s) * 16 + r) * 2] - m_max);
-      num = fmaf(w, ws_o[((part0 + s) * 16 + r) * rank + c], num);
-      den = fmaf(w, ws_ml[((part0 + s) * 16 + r) * 2 + 1], den);
+    for (int s = threadIdx.x; s < n_splits; s += kWave) m_max = fmaxf(m_max, ws_ml[((part0 + s) * 16 + r) * 2]);
+    m_max = wave_max(m_max);
+    float den = 0.f;
+    for (int s = threadIdx.x; s < n_splits; s += kWave) {
+      const float ws = exp2f(ws_ml[((part0 + s) * 16 + r) * 2] - m_max);
+      w[s] = ws;
+      den = fmaf(ws, ws_ml[((part0 + s) * 16 + r) * 2 + 1], den);
     }
-    out[(static_cast<size_t>(tok0 + tt) * n_heads + head) * rank + c] = num / den;
+    den = wave_sum(den);
+    if (threadIdx.x == 0) inv_den = 1.f / den;
+  }
+  __syncthreads();
+  float* o = out + (static_cast<size_t>(tok0 + tt) * n_heads + head) * rank;
+  for (int c = 4 * threadIdx.x; c < rank; c += 4 * blockDim.x) {
+    float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (s0 + j < n_splits) v[j] = *reinterpret_cast<const float4*>(ws_o + ((part0 + s0 + j) * 16 + r) * rank + c);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (s0 + j < n_splits) {
+          const float ws = w[s0 + j];
+          num.x = fmaf(ws, v[j].x, num.x); num.y = fmaf(ws, v[j].y, num.y);
+          num.z = fmaf(ws, v[j].z, num.z); num.w = fmaf(ws, v[j].w, num.w);
+        }
+    }
+    *reinterpret_cast<float4*>(o + c) = make_float4(num.x * inv_den, num.y * inv_den, num.z * inv_den, num.w * inv_den);
   }
 }
 
@@ -602,7 +605,7 @@ extern "C" int yk_latent_attention_mfma(const float* q_lat, const void* kpages, 
   YK_CASE(3, 4)
 #undef YK_CASE
   if (n_splits > 1) {
-    latent_attention_merge_kernel<<<dim3(n_tiles, chunks), 256, 0, stream>>>(ws_o, ws_ml, tiles, n_heads, kv_rank, n_splits, out);
+    latent_attention_merge_kernel<<<dim3(n_tiles, chunks, 16), 128, 0, stream>>>(ws_o, ws_ml, tiles, n_heads, kv_rank, n_splits, out);
     return yk_check_launch("latent_attention_merge");
   }
   return 0;

@@ -86,6 +86,127 @@ __global__ __launch_bounds__(256) void sandwich_norm_kernel(
   }
 }
 
+// The same for rows of up to 4,096 elements in 16-byte pieces, a thread holding up to four of them in
+// registers: everything a thread reads (the branch's slices, the residual, both norms' weights and
+// biases) is asked for before the first reduction, one round trip to memory instead of six.
+template <typename T>
+__device__ __forceinline__ float4 sn_load4(const T* p);
+template <>
+__device__ __forceinline__ float4 sn_load4<float>(const float* p) {
+  return *reinterpret_cast<const float4*>(p);
+}
+template <>
+__device__ __forceinline__ float4 sn_load4<bf16_t>(const bf16_t* p) {
+  const uint2 w = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                     __uint_as_float(w.y & 0xffff0000u));
+}
+template <typename T>
+__device__ __forceinline__ void sn_store4(T* p, float4 v);
+template <>
+__device__ __forceinline__ void sn_store4<float>(float* p, float4 v) {
+  *reinterpret_cast<float4*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void sn_store4<bf16_t>(bf16_t* p, float4 v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(v.x, v.y), pack_bf16x2(v.z, v.w));
+}
+
+constexpr int kSnPieces = 4;
+
+__device__ __forceinline__ NormStats piece_stats(const float4* v, const bool* has, int width, int center, float eps, float* scratch) {
+  float mean = 0.f;
+  if (center) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < kSnPieces; ++k)
+      if (has[k]) s += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+    mean = block_sum(s, scratch) / static_cast<float>(width);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < kSnPieces; ++k)
+    if (has[k]) {
+      const float a = v[k].x - mean, b = v[k].y - mean, c = v[k].z - mean, d = v[k].w - mean;
+      ss = fmaf(a, a, fmaf(b, b, fmaf(c, c, fmaf(d, d, ss))));
+    }
+  return {mean, 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(width) + eps)};
+}
+
+__device__ __forceinline__ float4 piece_norm(float4 v, NormStats st, float4 w, float4 b) {
+  return make_float4(fmaf((v.x - st.mean) * st.inv, w.x, b.x), fmaf((v.y - st.mean) * st.inv, w.y, b.y),
+                     fmaf((v.z - st.mean) * st.inv, w.z, b.z), fmaf((v.w - st.mean) * st.inv, w.w, b.w));
+}
+
+template <typename TS, typename TW, typename TO>
+__global__ __launch_bounds__(256) void sandwich_norm_vec_kernel(
+    float* __restrict__ residual, const TS* __restrict__ src, int n_splits, size_t split_stride, int round_sum,
+    const TW* __restrict__ wa, const TW* __restrict__ ba, float eps_a, int center_a, int has_post, float scale,
+    const TW* __restrict__ wb, const TW* __restrict__ bb, float eps_b, int center_b, int has_pre,
+    const int32_t* __restrict__ rows, TO* __restrict__ out, int width) {
+  __shared__ float scratch[17];
+  const size_t n = blockIdx.x;
+  const size_t r = rows != nullptr ? static_cast<size_t>(rows[n]) : n;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 br[kSnPieces], rs[kSnPieces], fwa[kSnPieces], fba[kSnPieces], fwb[kSnPieces], fbb[kSnPieces];
+  bool has[kSnPieces];
+#pragma unroll
+  for (int k = 0; k < kSnPieces; ++k) {
+    const int c = 4 * (threadIdx.x + 256 * k);
+    has[k] = c < width;
+    br[k] = rs[k] = fba[k] = fbb[k] = zero;
+    fwa[k] = fwb[k] = zero;
+    if (!has[k]) continue;
+    if (src != nullptr) {
+      for (int s0 = 0; s0 < n_splits; s0 += 8) {
+        float4 t[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (s0 + j < n_splits) t[j] = sn_load4<TS>(src + (s0 + j) * split_stride + r * width + c);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (s0 + j < n_splits) {
+            br[k].x += t[j].x; br[k].y += t[j].y; br[k].z += t[j].z; br[k].w += t[j].w;
+          }
+      }
+      br[k] = make_float4(as_output(br[k].x, round_sum), as_output(br[k].y, round_sum), as_output(br[k].z, round_sum),
+                          as_output(br[k].w, round_sum));
+    }
+    if (residual != nullptr) rs[k] = *reinterpret_cast<const float4*>(residual + r * width + c);
+    if (has_post) {
+      fwa[k] = sn_load4<TW>(wa + c);
+      if (ba != nullptr) fba[k] = sn_load4<TW>(ba + c);
+    }
+    if (has_pre) {
+      fwb[k] = sn_load4<TW>(wb + c);
+      if (bb != nullptr) fbb[k] = sn_load4<TW>(bb + c);
+    }
+  }
+  if (src != nullptr && has_post) {
+    const NormStats st = piece_stats(br, has, width, center_a, eps_a, scratch);
+#pragma unroll
+    for (int k = 0; k < kSnPieces; ++k) br[k] = piece_norm(br[k], st, fwa[k], fba[k]);
+  }
+  if (residual != nullptr) {
+#pragma unroll
+    for (int k = 0; k < kSnPieces; ++k) {
+      if (src != nullptr) {
+        rs[k] = make_float4(fmaf(scale, br[k].x, rs[k].x), fmaf(scale, br[k].y, rs[k].y), fmaf(scale, br[k].z, rs[k].z),
+                            fmaf(scale, br[k].w, rs[k].w));
+        if (rows == nullptr && has[k]) *reinterpret_cast<float4*>(residual + r * width + 4 * (threadIdx.x + 256 * k)) = rs[k];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < kSnPieces; ++k) rs[k] = br[k];
+  }
+  if (!has_pre) return;
+  const NormStats st = piece_stats(rs, has, width, center_b, eps_b, scratch);
+#pragma unroll
+  for (int k = 0; k < kSnPieces; ++k)
+    if (has[k]) sn_store4<TO>(out + n * width + 4 * (threadIdx.x + 256 * k), piece_norm(rs[k], st, fwb[k], fbb[k]));
+}
+
 // src_rows: rows of residual and of every slice of src (the stride between slices); n_rows: rows of out.
 extern "C" int yk_sandwich_norm(float* residual, const void* src, int src_dtype, int n_splits, int round_sum, int src_rows,
                                 const void* wa, const void* ba, float eps_a, int center_a, float scale, const void* wb,
@@ -100,8 +221,17 @@ extern "C" int yk_sandwich_norm(float* residual, const void* src, int src_dtype,
   if (n_rows == 0) return 0;
   const size_t stride = static_cast<size_t>(src_rows) * width;
   const size_t lds = (static_cast<size_t>(width) + 17) * sizeof(float);
+  auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = width % 4 == 0 && width <= 4 * 256 * kSnPieces && al(residual) && al(src) && al(wa) && al(ba) && al(wb) &&
+                   al(bb) && al(out);
 #define YK_CASE(SD, TS, WD, TW, OD, TO)                                                                           \
   if ((src == nullptr || src_dtype == SD) && w_dtype == WD && (out == nullptr || out_dtype == OD)) {              \
+    if (vec)                                                                                                      \
+      sandwich_norm_vec_kernel<TS, TW, TO><<<n_rows, 256, 0, stream>>>(                                           \
+          residual, static_cast<const TS*>(src), n_splits, stride, round_sum, static_cast<const TW*>(wa),         \
+          static_cast<const TW*>(ba), eps_a, center_a, wa != nullptr, scale, static_cast<const TW*>(wb),          \
+          static_cast<const TW*>(bb), eps_b, center_b, wb != nullptr, rows, static_cast<TO*>(out), width);        \
+    else                                                                                                          \
     sandwich_norm_kernel<TS, TW, TO><<<n_rows, 256, lds, stream>>>(                                               \
         residual, static_cast<const TS*>(src), n_splits, stride, round_sum, static_cast<const TW*>(wa),           \
         static_cast<const TW*>(ba), eps_a, center_a, wa != nullptr, scale, static_cast<const TW*>(wb),            \

@@ -29,11 +29,38 @@ constexpr int kScanTokens = 32;  // tokens staged at a time (fewer where LDS wou
 
 __device__ __forceinline__ float scan_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 
-// the sum over the TPC lanes of a column (lanes that differ in their low bits)
+// the sum over the TPC lanes of a column (lanes that differ in their low bits), in all of them.  Inside
+// a row of 16 lanes the exchanges are register moves (quad permutations, then rotations of the row by 4
+// and by 8: after the quads' sums, s_j = Q_j + Q_(j+1) and s_j + s_(j+2) is the row's sum); wider groups
+// go on through the LDS pipe.
+__device__ __forceinline__ float dpp_add(float v, int ctrl_xor1_2_ror4_8) {
+  const int x = __float_as_int(v);
+  int y;
+  switch (ctrl_xor1_2_ror4_8) {
+    case 0: y = __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xf, 0xf, false); break;   // quad_perm [1,0,3,2]
+    case 1: y = __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xf, 0xf, false); break;   // quad_perm [2,3,0,1]
+    case 2: y = __builtin_amdgcn_update_dpp(0, x, 0x124, 0xf, 0xf, false); break;  // row_ror:4
+    default: y = __builtin_amdgcn_update_dpp(0, x, 0x128, 0xf, 0xf, false); break; // row_ror:8
+  }
+  return v + __int_as_float(y);
+}
 template <int TPC>
 __device__ __forceinline__ float column_sum(float v) {
+  if (TPC >= 2) v = dpp_add(v, 0);
+  if (TPC >= 4) v = dpp_add(v, 1);
+  if (TPC == 8) {
+    // two quads a column: each takes the other's sum (quads 0 and 2 from four lanes up, 1 and 3 from four down)
+    const int x = __float_as_int(v);
+    int y = __builtin_amdgcn_update_dpp(0, x, 0x104, 0xf, 0x5, false);  // row_shl:4 into quads 0 and 2
+    y = __builtin_amdgcn_update_dpp(y, x, 0x114, 0xf, 0xa, false);      // row_shr:4 into quads 1 and 3
+    v += __int_as_float(y);
+  }
+  if (TPC >= 16) {
+    v = dpp_add(v, 2);
+    v = dpp_add(v, 3);
+  }
 #pragma unroll
-  for (int o = TPC / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  for (int o = 16; o < TPC; o <<= 1) v += __shfl_xor(v, o, kWave);
   return v;
 }
 
@@ -54,6 +81,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
   float* as = qs + chunk * DP;                            // [chunk][DP] (per channel) or [chunk]
   float* vs = as + chunk * (decay_mode == 1 ? DP : 1);    // [chunk][cols_per_block]
   float* bs = vs + chunk * cols_per_block;                // [chunk]
+  float* kqs = bs + chunk;                                // [chunk]: k . q of every token, as they enter the recurrence
 
   const int seq = blockIdx.x, h = blockIdx.y, kvh = h / (n_heads / n_kv);
   const int col0 = blockIdx.z * cols_per_block;
@@ -130,17 +158,30 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       bs[t] = delta ? 1.f / (1.f + expf(-beta[n * beta_stride + beta_col + h])) : 1.f;
     }
     __syncthreads();
-    if (unit_eps >= 0.f) {
-      // a wave per token and vector: the sum of squares over the wave, the row scaled where it lies
-      for (int item = wave; item < 2 * nt; item += n_waves) {
-        float* row = ((item & 1) ? ks : qs) + (item >> 1) * DP;
-        float ss = 0.f;
-        for (int c = lane; c < DP; c += kWave) ss = fmaf(row[c], row[c], ss);
-        const float mul = ((item & 1) ? 1.f : q_scale) / sqrtf(wave_sum(ss) + unit_eps);
-        for (int c = lane; c < DP; c += kWave) row[c] *= mul;
+    // a wave per token: unit norms (the rows scaled where they lie) and k . q, which the read-out needs
+    for (int t = wave; t < nt; t += n_waves) {
+      float* qrow = qs + t * DP;
+      float* krow = ks + t * DP;
+      float ssq = 0.f, ssk = 0.f, dot = 0.f;
+      for (int c = lane; c < DP; c += kWave) {
+        const float a = qrow[c], b = krow[c];
+        ssq = fmaf(a, a, ssq);
+        ssk = fmaf(b, b, ssk);
+        dot = fmaf(a, b, dot);
       }
-      __syncthreads();
+      dot = wave_sum(dot);
+      if (unit_eps >= 0.f) {
+        const float mq = q_scale / sqrtf(wave_sum(ssq) + unit_eps), mk = 1.f / sqrtf(wave_sum(ssk) + unit_eps);
+        for (int c = lane; c < DP; c += kWave) {
+          qrow[c] *= mq;
+          krow[c] *= mk;
+        }
+        dot *= mq * mk;
+      }
+      if (lane == 0) kqs[t] = dot;
     }
+    __syncthreads();
+#pragma unroll 2
     for (int t = 0; t < nt; ++t) {
       const float4* kt = reinterpret_cast<const float4*>(ks + t * DP + sub * kScanRows);
       const float4* qt = reinterpret_cast<const float4*>(qs + t * DP + sub * kScanRows);
@@ -162,29 +203,26 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
 #pragma unroll
         for (int r = 0; r < kScanRows; ++r) S[r] *= a;
       }
-      float u = vs[t * cols_per_block + col_local];
-      if (delta) {
-        // S^T k in four partial sums (rows r, r + 4, ...), then over the column's lanes
-        float p[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int r = 0; r < kScanRows; ++r) p[r % 4] = fmaf(S[r], kr[r], p[r % 4]);
-        const float sk = column_sum<TPC>((p[0] + p[1]) + (p[2] + p[3]));
-        u = bs[t] * (u - sk);
-      }
-      float p[4] = {0.f, 0.f, 0.f, 0.f};
+      // both sums over the decayed S at once: S^T k for the write, S^T q for the read-out, which sees the
+      // token's own write through q . (k u^T) = u (k . q)
+      float pk[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
+      float qr[kScanRows];
 #pragma unroll
       for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
         const float4 q4 = qt[r4];
-        S[4 * r4] = fmaf(kr[4 * r4], u, S[4 * r4]);
-        S[4 * r4 + 1] = fmaf(kr[4 * r4 + 1], u, S[4 * r4 + 1]);
-        S[4 * r4 + 2] = fmaf(kr[4 * r4 + 2], u, S[4 * r4 + 2]);
-        S[4 * r4 + 3] = fmaf(kr[4 * r4 + 3], u, S[4 * r4 + 3]);
-        p[0] = fmaf(S[4 * r4], q4.x, p[0]);
-        p[1] = fmaf(S[4 * r4 + 1], q4.y, p[1]);
-        p[2] = fmaf(S[4 * r4 + 2], q4.z, p[2]);
-        p[3] = fmaf(S[4 * r4 + 3], q4.w, p[3]);
+        qr[4 * r4] = q4.x; qr[4 * r4 + 1] = q4.y; qr[4 * r4 + 2] = q4.z; qr[4 * r4 + 3] = q4.w;
       }
-      const float so = column_sum<TPC>((p[0] + p[1]) + (p[2] + p[3]));
+#pragma unroll
+      for (int r = 0; r < kScanRows; ++r) {
+        pk[r % 4] = fmaf(S[r], kr[r], pk[r % 4]);
+        pq[r % 4] = fmaf(S[r], qr[r], pq[r % 4]);
+      }
+      const float sq = column_sum<TPC>((pq[0] + pq[1]) + (pq[2] + pq[3]));
+      float u = vs[t * cols_per_block + col_local];
+      if (delta) u = bs[t] * (u - column_sum<TPC>((pk[0] + pk[1]) + (pk[2] + pk[3])));
+      const float so = fmaf(u, kqs[t], sq);
+#pragma unroll
+      for (int r = 0; r < kScanRows; ++r) S[r] = fmaf(kr[r], u, S[r]);
       if (has_col && sub == 0) out[(static_cast<size_t>(q0 + t0 + t) * n_heads + h) * vdim + col] = so;
     }
   }
@@ -221,7 +259,7 @@ extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, 
   dim3 grid(n_seqs, n_heads, (vdim + cols - 1) / cols);
   const size_t dp = static_cast<size_t>(tpc) * kScanRows;
   int chunk = kScanTokens;
-  const size_t per_token = sizeof(float) * (2 * dp + (decay_mode == 1 ? dp : 1) + cols + 1);
+  const size_t per_token = sizeof(float) * (2 * dp + (decay_mode == 1 ? dp : 1) + cols + 2);
   while (chunk > 4 && chunk * per_token > 100 * 1024) chunk /= 2;
   const size_t lds = chunk * per_token;
   YK_REQUIRE(lds <= 128 * 1024, "linear_state_scan: the staged tokens do not fit in LDS");

@@ -102,10 +102,9 @@ _SIGNATURES = {
     ),
     "yk_head_linear": (
         [_vp, _c_int, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int,
-         _c_int, _vp],
+         _c_int, _c_int, _vp],
         _c_int,
     ),
-    "yk_head_linear_out": ([_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_latent_tile_tokens": ([_c_int], _c_int),
     "yk_latent_attention": ([_vp, _vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp], _c_int),
     "yk_linear_state_scan": (
@@ -1390,23 +1389,16 @@ class HipOps:
             self._rows(gate, "head_linear gate")
             if gate.shape[0] != n or gate.shape[1] < gate_col + n_heads:
                 raise KernelError("head_linear: the gate's rows do not hold a column per head")
-        if x.dtype == torch.float32 and tail == 0 and (gate is None or gate.dtype == out_dtype):
-            self._check(self.lib.yk_head_linear_out(
-                x.data_ptr(), x.stride(0), w.data_ptr(), _code(w.dtype), out.data_ptr(), _code(out_dtype), n_heads, in_dim, out_dim,
-                _ptr(gate), 0 if gate is None else gate.stride(0), gate_col, n, self._stream()))
-            return out
         cos = sin = None
         inter = 0
         if tail:
             if rotation is None or rotation.rotary_dim != tail or positions is None:
                 raise KernelError("head_linear: the tail needs a rotation that covers it exactly, and positions")
             cos, sin, inter = rotation.cos, rotation.sin, int(rotation.interleaved)
-        if gate is not None and gate.dtype != x.dtype:
-            raise KernelError("head_linear: gate and input differ in dtype")
         self._check(self.lib.yk_head_linear(
             x.data_ptr(), x.stride(0), _code(x.dtype), w.data_ptr(), _code(w.dtype), out.data_ptr(), _code(out_dtype), n_heads, in_dim,
-            out_dim, tail, _ptr(positions), _ptr(cos), _ptr(sin), inter, _ptr(gate), 0 if gate is None else gate.stride(0), gate_col,
-            n, self._stream()))
+            out_dim, tail, _ptr(positions), _ptr(cos), _ptr(sin), inter, _ptr(gate), 0 if gate is None else _code(gate.dtype),
+            0 if gate is None else gate.stride(0), gate_col, n, self._stream()))
         return out
 
     def latent_attention_on_matrix_cores(self, act_dtype: torch.dtype, kv_rank: int, rot_dim: int, page_size: int) -> bool:
