@@ -493,7 +493,7 @@ def latent_prepare(proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, ro
     return c_q
 
 
-def head_linear(x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0):
+def head_linear(x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0, w_t=None):
     """Per head, out[n, h, :out_dim] = x[n, h, :in_dim] . w[h] (w [heads, in, out]); ``tail`` more elements of
     every head of x follow the product, turned by the token's position; ``gate``: the head's output times
     the sigmoid of column gate_col + h of ``gate``."""

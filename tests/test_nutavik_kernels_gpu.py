@@ -195,6 +195,31 @@ def test_one_row_stands_out_at_every_border(dtype, heads, kv_rank, rot_dim, spec
         assert (got[seen].view(len(seen), heads, kv_rank)[:, :, 0].cpu() > 20.0).all()
 
 
+@pytest.mark.parametrize("heads,in_dim,out_dim,tail,n", [(3, 32, 48, 8, 40), (16, 128, 512, 64, 150), (5, 512, 128, 0, 77), (2, 64, 16, 16, 33)])
+def test_head_linear_on_matrix_cores(heads, in_dim, out_dim, tail, n):
+    """Many tokens, bfloat16 weights kept transposed: into the latent (bfloat16 in, a turned tail, float32
+    out) and out of it (float32 in, rounded as it is loaded, gates, bfloat16 out); token tiles that end
+    inside a wave's 16 rows, column tiles that end inside a workgroup's 64."""
+    o = ops()
+    g = torch.Generator().manual_seed(n)
+    bf = torch.bfloat16
+    w = (torch.randn(heads, in_dim, out_dim, generator=g) / in_dim ** 0.5).to(bf)
+    w_t = o.head_weights_transposed(w.cuda())
+    assert w_t is not None and tuple(w_t.shape) == (heads, out_dim, in_dim)
+    pos = torch.randint(0, 64, (n,), generator=g, dtype=torch.int32)
+    rot = rotation(tail, 64) if tail else None
+    x = torch.randn(n, heads * (in_dim + tail), generator=g).to(bf)
+    want = R.head_linear(x, w, heads, in_dim, out_dim, torch.float32, tail=tail, rotation=rot, positions=pos)
+    got = o.head_linear(x.cuda(), w.cuda(), heads, in_dim, out_dim, torch.float32, tail=tail, rotation=on_device(rot) if tail else None,
+                        positions=pos.cuda(), w_t=w_t)
+    close(got, want, torch.float32, "into the latent", f32=2e-5)
+    xo = torch.randn(n, heads * in_dim, generator=g).to(bf).float()  # (values bfloat16 holds: the rounding at the load is exact)
+    gate = torch.randn(n, heads + 11, generator=g).to(bf)
+    want = R.head_linear(xo, w, heads, in_dim, out_dim, bf, gate=gate, gate_col=7)
+    got = o.head_linear(xo.cuda(), w.cuda(), heads, in_dim, out_dim, bf, gate=gate.cuda(), gate_col=7, w_t=w_t)
+    close(got, want, bf, "out of the latent", bf16=1e-2)
+
+
 @pytest.mark.parametrize("heads,kv_rank,rot_dim,page", [(2, 64, 32, 32), (5, 128, 32, 64), (16, 512, 64, 64), (20, 256, 64, 32)])
 @pytest.mark.parametrize("special", [0, 31, 32, 63, 64, 399, 400])
 @pytest.mark.parametrize("splits", [1, 3, None])

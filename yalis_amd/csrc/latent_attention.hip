@@ -177,7 +177,7 @@ extern "C" int yk_head_linear(const void* x, int x_stride, int x_dtype, const vo
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && in_dim > 0 && out_dim > 0 && tail >= 0 && tail % 2 == 0, "head_linear: bad sizes");
   YK_REQUIRE(x_stride >= n_heads * (in_dim + tail), "head_linear: the input's rows are shorter than its heads");
   YK_REQUIRE(tail == 0 || (positions != nullptr && cos_t != nullptr && sin_t != nullptr), "head_linear: a turned tail needs positions and tables");
-  const int slices = n_tokens > 4 * kHeadTokens ? 1 : 4;
+  const int slices = 4;
   const size_t lds = sizeof(float) * (static_cast<size_t>(kHeadTokens) * (in_dim + tail) + slices * kHeadTokens * kHeadOut);
   YK_REQUIRE(lds <= 64 * 1024, "head_linear: heads of more than 1,700 input elements do not fit");
   if (n_tokens == 0) return 0;
@@ -205,6 +205,117 @@ extern "C" int yk_head_linear(const void* x, int x_stride, int x_dtype, const vo
   YK_CASE(YK_F32, float, YK_F32, float, YK_BF16, bf16_t, YK_BF16, bf16_t)
 #undef YK_CASE
   return yk_fail("head_linear: unsupported dtype combination");
+}
+
+// The same products on the matrix cores, for many tokens: bfloat16 weights kept [heads][out][in] (a row of
+// the second operand is then 16 bytes of memory a lane), the input bfloat16 or float32 (rounded as it is
+// loaded).  A wave makes 16 tokens x 64 columns of one head: the first operand is 16 input rows x 32
+// elements, loaded as it lies there.  Four waves a workgroup take four token tiles.
+typedef __bf16 hl_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float hl_f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t hl_u32x4_t __attribute__((ext_vector_type(4)));
+union HlFrag {
+  hl_u32x4_t u;
+  hl_bf16x8_t v;
+};
+
+template <typename TX>
+__device__ __forceinline__ hl_u32x4_t hl_load8(const TX* p);
+template <>
+__device__ __forceinline__ hl_u32x4_t hl_load8<bf16_t>(const bf16_t* p) {
+  return *reinterpret_cast<const hl_u32x4_t*>(p);
+}
+template <>
+__device__ __forceinline__ hl_u32x4_t hl_load8<float>(const float* p) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  return hl_u32x4_t{pack_bf16x2(a.x, a.y), pack_bf16x2(a.z, a.w), pack_bf16x2(b.x, b.y), pack_bf16x2(b.z, b.w)};
+}
+
+template <typename TX, typename TG, typename TO>
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(
+    const TX* __restrict__ x, int x_stride, const bf16_t* __restrict__ w_t, TO* __restrict__ out, int out_stride, int in_dim,
+    int out_dim, int tail, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int interleaved, const TG* __restrict__ gate, int gate_stride, int gate_col,
+    int n_tokens) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int r = lane % 16, g = lane / 16;
+  const int n0 = (blockIdx.x * 4 + wave) * 16, h = blockIdx.y, o0 = blockIdx.z * 64;
+  if (n0 >= n_tokens) return;
+  const int xw = in_dim + tail, ow = out_dim + tail;
+  const int tok = min(n0 + r, n_tokens - 1);  // (rows past the end repeat the last token and are not stored)
+  const TX* xp = x + static_cast<size_t>(tok) * x_stride + h * xw + 8 * g;
+  const bf16_t* wp = w_t + (static_cast<size_t>(h) * out_dim + o0 + r) * in_dim + 8 * g;
+  hl_f32x4_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = hl_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int n_tiles = min(4, (out_dim - o0) / 16);
+  for (int k0 = 0; k0 < in_dim; k0 += 32) {
+    HlFrag a;
+    a.u = hl_load8<TX>(xp + k0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (j < n_tiles) {
+        HlFrag b;
+        b.u = *reinterpret_cast<const hl_u32x4_t*>(wp + static_cast<size_t>(16 * j) * in_dim + k0);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[j], 0, 0, 0);
+      }
+    }
+  }
+  // acc[j][i]: token n0 + 4 g + i, column o0 + 16 j + r
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n0 + 4 * g + i;
+    if (n >= n_tokens) continue;
+    float gv = 1.f;
+    if (gate != nullptr) gv = 1.f / (1.f + expf(-to_f32<TG>(gate[static_cast<size_t>(n) * gate_stride + gate_col + h])));
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (j < n_tiles) out[static_cast<size_t>(n) * out_stride + h * ow + o0 + 16 * j + r] = from_f32<TO>(acc[j][i] * gv);
+  }
+  if (blockIdx.z != 0 || tail == 0) return;
+  const int half = tail / 2;
+  for (int i = lane; i < 16 * half; i += kWave) {
+    const int t = i / half, j = i % half, n = n0 + t;
+    if (n >= n_tokens) break;
+    const int ia = interleaved ? 2 * j : j, ib = interleaved ? 2 * j + 1 : j + half;
+    const TX* src = x + static_cast<size_t>(n) * x_stride + h * xw + in_dim;
+    const float a = to_f32<TX>(src[ia]), b = to_f32<TX>(src[ib]);
+    const size_t p = static_cast<size_t>(positions[n]);
+    const float c = cos_t[p * half + j], sn = sin_t[p * half + j];
+    TO* dst = out + static_cast<size_t>(n) * out_stride + h * ow + out_dim;
+    dst[ia] = from_f32<TO>(rot_first(a, b, c, sn));
+    dst[ib] = from_f32<TO>(rot_second(a, b, c, sn));
+  }
+}
+
+extern "C" int yk_head_linear_mfma_ok(int in_dim, int out_dim, int tail) { return in_dim % 32 == 0 && out_dim % 16 == 0 && tail % 8 == 0; }
+
+// w_t: bfloat16 [heads][out_dim][in_dim]; x bfloat16 or float32 with 16-byte aligned rows and heads
+extern "C" int yk_head_linear_mfma(const void* x, int x_stride, int x_dtype, const void* w_t, void* out, int out_dtype, int n_heads,
+                                   int in_dim, int out_dim, int tail, const int32_t* positions, const float* cos_t,
+                                   const float* sin_t, int interleaved, const void* gate, int gate_dtype, int gate_stride,
+                                   int gate_col, int n_tokens, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && yk_head_linear_mfma_ok(in_dim, out_dim, tail), "head_linear_mfma: sizes it is not built for");
+  YK_REQUIRE(x_stride >= n_heads * (in_dim + tail) && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(w_t) % 16 == 0,
+             "head_linear_mfma: the input's rows must be 16-byte aligned");
+  YK_REQUIRE(tail == 0 || (positions != nullptr && cos_t != nullptr && sin_t != nullptr), "head_linear_mfma: a turned tail needs positions and tables");
+  if (n_tokens == 0) return 0;
+  dim3 grid((n_tokens + 63) / 64, n_heads, (out_dim + 63) / 64);
+  const int out_stride = n_heads * (out_dim + tail);
+  if (gate == nullptr) gate_dtype = out_dtype;
+#define YK_CASE(XD, TX, GD, TG, OD, TO)                                                                                 \
+  if (x_dtype == XD && gate_dtype == GD && out_dtype == OD) {                                                           \
+    head_linear_mfma_kernel<TX, TG, TO><<<grid, 256, 0, stream>>>(                                                      \
+        static_cast<const TX*>(x), x_stride, static_cast<const bf16_t*>(w_t), static_cast<TO*>(out), out_stride, in_dim, \
+        out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TG*>(gate), gate_stride, gate_col,       \
+        n_tokens);                                                                                                      \
+    return yk_check_launch("head_linear_mfma");                                                                         \
+  }
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_BF16, bf16_t)
+#undef YK_CASE
+  return yk_fail("head_linear_mfma: unsupported dtype combination");
 }
 
 // --------------------------------------------------------------------------------- attention

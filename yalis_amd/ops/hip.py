@@ -105,6 +105,12 @@ _SIGNATURES = {
          _c_int, _c_int, _vp],
         _c_int,
     ),
+    "yk_head_linear_mfma_ok": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_head_linear_mfma": (
+        [_vp, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int,
+         _c_int, _c_int, _vp],
+        _c_int,
+    ),
     "yk_latent_tile_tokens": ([_c_int], _c_int),
     "yk_latent_attention": ([_vp, _vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp], _c_int),
     "yk_linear_state_scan": (
@@ -1375,11 +1381,23 @@ class HipOps:
             self._stream()))
         return c_q
 
-    def head_linear(self, x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0):
+    # tokens from which the per-head products run on the matrix cores (where sizes and types allow)
+    HEAD_LINEAR_MFMA_FROM = 33
+
+    def head_weights_transposed(self, w: torch.Tensor) -> Optional[torch.Tensor]:
+        """What ``head_linear`` takes as ``w_t``: the weights [heads, in, out] once more as [heads, out, in],
+        where the matrix-core form may use them (bfloat16, sizes it is built for); else None."""
+        if w.dtype != torch.bfloat16 or w.dim() != 3 or not self._ask("yk_head_linear_mfma_ok", w.shape[1], w.shape[2], 0):
+            return None
+        return w.transpose(1, 2).contiguous()
+
+    def head_linear(self, x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0,
+                    w_t=None):
         """Per head, out[n, h, :out_dim] = x[n, h, :in_dim] . w[h] with w [heads, in_dim, out_dim]
         (float32 sums).  ``tail`` further elements of every head of x follow the product in the output,
         turned by the token's position (``rotation``, ``positions``); ``gate`` [N, >= gate_col + heads]:
-        head h's output is multiplied by sigmoid(gate[n, gate_col + h])."""
+        head h's output is multiplied by sigmoid(gate[n, gate_col + h]).  ``w_t`` (``head_weights_transposed``):
+        with it, products of many tokens run on the matrix cores (the input rounded to bfloat16 there)."""
         self._rows(x, "head_linear input")
         n = x.shape[0]
         if tuple(w.shape) != (n_heads, in_dim, out_dim) or not w.is_contiguous() or x.shape[1] != n_heads * (in_dim + tail):
@@ -1395,6 +1413,17 @@ class HipOps:
             if rotation is None or rotation.rotary_dim != tail or positions is None:
                 raise KernelError("head_linear: the tail needs a rotation that covers it exactly, and positions")
             cos, sin, inter = rotation.cos, rotation.sin, int(rotation.interleaved)
+        gate_ok = gate is None or (gate.dtype == out_dtype if x.dtype == torch.float32 else False)
+        if (w_t is not None and n >= self.HEAD_LINEAR_MFMA_FROM and tuple(w_t.shape) == (n_heads, out_dim, in_dim) and w_t.is_contiguous()
+                and w_t.dtype == torch.bfloat16 and self._ask("yk_head_linear_mfma_ok", in_dim, out_dim, tail)
+                and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and (in_dim + tail) % 8 == 0 and gate_ok
+                and ((x.dtype, out_dtype) in ((torch.bfloat16, torch.float32), (torch.float32, torch.bfloat16)))
+                and (x.dtype == torch.float32 or gate is None)):
+            self._check(self.lib.yk_head_linear_mfma(
+                x.data_ptr(), x.stride(0), _code(x.dtype), w_t.data_ptr(), out.data_ptr(), _code(out_dtype), n_heads, in_dim, out_dim,
+                tail, _ptr(positions), _ptr(cos), _ptr(sin), inter, _ptr(gate), 0 if gate is None else _code(gate.dtype),
+                0 if gate is None else gate.stride(0), gate_col, n, self._stream()))
+            return out
         self._check(self.lib.yk_head_linear(
             x.data_ptr(), x.stride(0), _code(x.dtype), w.data_ptr(), _code(w.dtype), out.data_ptr(), _code(out_dtype), n_heads, in_dim,
             out_dim, tail, _ptr(positions), _ptr(cos), _ptr(sin), inter, _ptr(gate), 0 if gate is None else _code(gate.dtype),

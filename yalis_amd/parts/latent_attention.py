@@ -67,7 +67,7 @@ class LatentAttention(Mixer):
         names = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o"}
         names.update(params.get("names", {}))
         self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
-        self.w_down = self.w_qn = self.w_kvn = self.w_uq = self.w_uk = self.w_uv_t = self.w_o = None
+        self.w_down = self.w_qn = self.w_kvn = self.w_uq = self.w_uk = self.w_uv_t = self.w_o = self.w_uk_t = self.w_uv = None
         # columns of the stacked down-projection: [dq | dkv (where the layer keeps a cache) | gates], each
         # section starting at a multiple of 8
         up8 = lambda n: n + (-n % 8)
@@ -115,6 +115,10 @@ class LatentAttention(Mixer):
         self.w_uk = tensors[n["uk"]].view(H, self.head_dim, self.kv_rank).contiguous()
         self.w_uv_t = tensors[n["uv"]].view(H, self.value_dim, self.kv_rank).transpose(1, 2).contiguous()
         self.w_o = tensors[n["o"]]
+        # the same weights [head][out][in] where the kernel library's matrix-core products want them
+        transposed = getattr(self.rt.ops, "head_weights_transposed", None)
+        self.w_uk_t = transposed(self.w_uk) if transposed is not None else None
+        self.w_uv = transposed(self.w_uv_t) if transposed is not None else None
 
     def kv_need(self) -> KVNeed:
         # one row of kv_rank + rot_dim elements per token and no values: the row serves as both
@@ -143,9 +147,9 @@ class LatentAttention(Mixer):
         q = ops.linear(c_q, self.w_uq, act)
         # queries in the latent's space: [W_uk^T q[:dim] | q[dim:] turned by the position], float32
         q_lat = ops.head_linear(q, self.w_uk, self.n_heads, self.head_dim, self.kv_rank, torch.float32, tail=self.rot_dim,
-                                rotation=self.rotation, positions=ctx.arrays["positions"])
+                                rotation=self.rotation, positions=ctx.arrays["positions"], w_t=self.w_uk_t)
         o_lat = ops.latent_attention(q_lat, pages, self.n_heads, self.kv_rank, self.rot_dim, self.scale, ctx, site.group,
                                      self.rt.page_size, tiles=ctx.arrays[f"latent_tiles_{self.tile_tokens}"], values=values)
         o = ops.head_linear(o_lat, self.w_uv_t, self.n_heads, self.kv_rank, self.value_dim, act,
-                            gate=proj if self.gate_name else None, gate_col=self.gate_col)
+                            gate=proj if self.gate_name else None, gate_col=self.gate_col, w_t=self.w_uv)
         return ops.linear(o, self.w_o, act, partial_ok=True)
