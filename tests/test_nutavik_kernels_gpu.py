@@ -292,7 +292,7 @@ def test_convolution_with_silu_and_its_state(dtype, taps):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("kind", ["delta", "gla"])
-@pytest.mark.parametrize("heads,kv,dim,vdim", [(4, 2, 12, 10), (2, 2, 24, 9), (2, 2, 64, 32), (3, 1, 128, 70), (1, 1, 200, 5), (2, 1, 16, 300), (1, 1, 300, 40)])
+@pytest.mark.parametrize("heads,kv,dim,vdim", [(4, 2, 12, 10), (2, 2, 24, 9), (2, 2, 64, 32), (3, 1, 128, 70), (1, 1, 200, 5), (2, 1, 16, 300), (1, 1, 300, 40), (2, 1, 8, 20), (1, 1, 600, 6)])
 def test_linear_state_scan(dtype, kind, heads, kv, dim, vdim):
     """Both kinds of write and of decay, key channels from fewer than a lane's share to many lanes a
     column, more value columns than a workgroup holds; spans of one token and of several staged chunks,

@@ -24,7 +24,7 @@
 
 #include "common.h"
 
-constexpr int kScanRows = 16;    // rows of S a lane holds: sub * 16 .. sub * 16 + 15 of its column
+constexpr int kScanRowsMax = 16;  // rows of S a lane holds at the most (template R: 8 or 16): sub * R .. sub * R + R - 1 of its column
 constexpr int kScanTokens = 32;  // tokens staged at a time (fewer where LDS would not hold them)
 
 __device__ __forceinline__ float scan_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
@@ -59,14 +59,37 @@ __device__ __forceinline__ float column_sum(float v) {
     v = dpp_add(v, 2);
     v = dpp_add(v, 3);
   }
-#pragma unroll
-  for (int o = 16; o < TPC; o <<= 1) v += __shfl_xor(v, o, kWave);
+  if (TPC >= 32) {  // lanes r and r + 16
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  }
+  if (TPC >= 64) {  // and the other half of the wave
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(b[0]) + __uint_as_float(b[1]);
+  }
   return v;
+}
+
+// eight consecutive elements (16-byte aligned where T is bfloat16, 32 where float) as floats
+template <typename T>
+__device__ __forceinline__ void scan_load8(const T* p, float* out);
+template <>
+__device__ __forceinline__ void scan_load8<float>(const float* p, float* out) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w; out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+}
+template <>
+__device__ __forceinline__ void scan_load8<bf16_t>(const bf16_t* p, float* out) {
+  const uint4 w = *reinterpret_cast<const uint4*>(p);
+  out[0] = __uint_as_float(w.x << 16); out[1] = __uint_as_float(w.x & 0xffff0000u);
+  out[2] = __uint_as_float(w.y << 16); out[3] = __uint_as_float(w.y & 0xffff0000u);
+  out[4] = __uint_as_float(w.z << 16); out[5] = __uint_as_float(w.z & 0xffff0000u);
+  out[6] = __uint_as_float(w.w << 16); out[7] = __uint_as_float(w.w & 0xffff0000u);
 }
 
 // LDS per staged token: k and q padded to TPC * 16 floats each (rows past dim are zeros, so nobody
 // asks whether a row exists), the per-channel decays likewise where there are any
-template <typename T, int TPC>
+template <typename T, int TPC, int kScanRows, bool VEC>
 __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     const T* __restrict__ qkv, int qkv_stride, int n_heads, int n_kv, int dim, int vdim, float* __restrict__ state,
     const int32_t* __restrict__ seq_qstart, const int32_t* __restrict__ seq_qlen, const int32_t* __restrict__ state_slots,
@@ -75,11 +98,12 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     int beta_stride, int beta_col, int chunk, float* __restrict__ out) {
   extern __shared__ float lds[];
   constexpr int DP = TPC * kScanRows;  // padded key channels
+  constexpr int DS = DP + 4;           // a staged row's stride: rows of different tokens then start in different banks
   const int cols_per_block = blockDim.x / TPC;
-  float* ks = lds;                                        // [chunk][DP]
-  float* qs = ks + chunk * DP;                            // [chunk][DP]
-  float* as = qs + chunk * DP;                            // [chunk][DP] (per channel) or [chunk]
-  float* vs = as + chunk * (decay_mode == 1 ? DP : 1);    // [chunk][cols_per_block]
+  float* ks = lds;                                        // [chunk][DS]
+  float* qs = ks + chunk * DS;                            // [chunk][DS]
+  float* as = qs + chunk * DS;                            // [chunk][DS] (per channel) or [chunk]
+  float* vs = as + chunk * (decay_mode == 1 ? DS : 1);    // [chunk][cols_per_block]
   float* bs = vs + chunk * cols_per_block;                // [chunk]
   float* kqs = bs + chunk;                                // [chunk]: k . q of every token, as they enter the recurrence
 
@@ -102,6 +126,100 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
   for (int t0 = 0; t0 < ql; t0 += chunk) {
     const int nt = min(chunk, ql - t0);
     __syncthreads();  // the chunk before has been read
+    if constexpr (VEC) {
+      // Everything the chunk needs is asked for at once, 16 bytes a load, before anything is used: q and
+      // k (eight elements a piece), the decays' logits and biases (four), v, the scalars.  One round
+      // trip to memory a chunk; one after the other the loads cost a round trip each, which was most
+      // of the kernel's time.
+      constexpr int P8 = DP / 8 > 0 ? DP / 8 : 1;  // pieces of a padded row (DP >= 16: at least two)
+      const float q_mul = unit_eps >= 0.f ? 1.f : q_scale;
+      const int n_qk = 2 * nt * (DP / 8);
+      float qk[8][8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int v = threadIdx.x + j * 256;
+        const int item = v / P8, c = 8 * (v % P8), t = item >> 1, is_k = item & 1;
+        if (v < n_qk && c < dim)
+          scan_load8<T>(qkv + static_cast<size_t>(q0 + t0 + t) * qkv_stride + (is_k ? kd : 0) + kvh * dim + c, qk[j]);
+        else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) qk[j][e] = 0.f;
+        }
+      }
+      constexpr int P4 = DP / 4;
+      const int n_dec = decay_mode == 1 ? nt * P4 : 0;
+      float4 dz[8], db[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int v = threadIdx.x + j * 256;
+        const int t = v / P4, c = 4 * (v % P4);
+        dz[j] = db[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < n_dec && c < dim) {
+          dz[j] = *reinterpret_cast<const float4*>(decay + static_cast<size_t>(q0 + t0 + t) * decay_stride + decay_col + h * dim + c);
+          db[j] = *reinterpret_cast<const float4*>(decay_p0 + h * dim + c);
+        }
+      }
+      const int n_v = nt * cols_per_block;
+      float vv[8];
+      for (int i0 = 0; i0 < n_v; i0 += 8 * 256) {  // (one pass unless a column is a single lane's)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = i0 + threadIdx.x + j * 256;
+          const int t = i / cols_per_block, c = col0 + i % cols_per_block;
+          vv[j] = i < n_v && c < vdim ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + 2 * kd + h * vdim + c]) : 0.f;
+        }
+        if (i0 + 8 * 256 < n_v) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int i = i0 + threadIdx.x + j * 256;
+            if (i < n_v) vs[i] = vv[j];
+          }
+        }
+      }
+      float s_dec = 0.f, s_beta = 0.f;
+      if (threadIdx.x < nt) {
+        const size_t n = static_cast<size_t>(q0 + t0 + threadIdx.x);
+        if (decay_mode == 0) s_dec = decay[n * decay_stride + decay_col + h];
+        if (delta) s_beta = beta[n * beta_stride + beta_col + h];
+      }
+      // ---- everything is on its way; now the stores
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int v = threadIdx.x + j * 256;
+        if (v < n_qk) {
+          const int item = v / P8, c = 8 * (v % P8), t = item >> 1, is_k = item & 1;
+          const float mul = is_k ? 1.f : q_mul;
+          float* dst = (is_k ? ks : qs) + t * DS + c;
+          *reinterpret_cast<float4*>(dst) = make_float4(qk[j][0] * mul, qk[j][1] * mul, qk[j][2] * mul, qk[j][3] * mul);
+          *reinterpret_cast<float4*>(dst + 4) = make_float4(qk[j][4] * mul, qk[j][5] * mul, qk[j][6] * mul, qk[j][7] * mul);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int v = threadIdx.x + j * 256;
+        if (v < n_dec) {
+          const int c = 4 * (v % P4);
+          // sigmoid(z)^(1/tau); channels past dim decay to nothing (their rows of S are zeros anyway)
+          float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (c < dim)
+            a = make_float4(expf(-scan_softplus(-(dz[j].x + db[j].x)) / tau), expf(-scan_softplus(-(dz[j].y + db[j].y)) / tau),
+                            expf(-scan_softplus(-(dz[j].z + db[j].z)) / tau), expf(-scan_softplus(-(dz[j].w + db[j].w)) / tau));
+          *reinterpret_cast<float4*>(as + (v / P4) * DS + c) = a;
+        }
+      }
+      {
+        const int i0 = (n_v - 1) / (8 * 256) * (8 * 256);  // the last pass's values are still in registers
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = i0 + threadIdx.x + j * 256;
+          if (i < n_v) vs[i] = vv[j];
+        }
+      }
+      if (threadIdx.x < nt) {
+        if (decay_mode == 0) as[threadIdx.x] = expf(-expf(decay_p0[h]) * scan_softplus(s_dec + decay_p1[h]));
+        bs[threadIdx.x] = delta ? 1.f / (1.f + expf(-s_beta)) : 1.f;
+      }
+    } else {
     // q and k of the chunk's tokens to LDS, every load of a thread asked for before the first is used
     // (one after the other they cost a round trip to memory each)
     {
@@ -122,7 +240,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
           const int i = i0 + j * blockDim.x;
           if (i < total) {
             const int item = i / DP, c = i % DP, t = item >> 1, is_k = item & 1;
-            ((is_k ? ks : qs) + t * DP)[c] = is_k ? x[j] : x[j] * q_mul;
+            ((is_k ? ks : qs) + t * DS)[c] = is_k ? x[j] : x[j] * q_mul;
           }
         }
       }
@@ -143,7 +261,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
         for (int j = 0; j < 8; ++j) {
           const int i = i0 + j * blockDim.x;
           // sigmoid(z)^(1/tau); channels past dim decay to nothing (their rows of S are zeros anyway)
-          if (i < total) as[i] = i % DP < dim ? expf(-scan_softplus(-z[j]) / tau) : 0.f;
+          if (i < total) as[(i / DP) * DS + i % DP] = i % DP < dim ? expf(-scan_softplus(-z[j]) / tau) : 0.f;
         }
       }
     }
@@ -157,70 +275,87 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
         as[t] = expf(-expf(decay_p0[h]) * scan_softplus(decay[n * decay_stride + decay_col + h] + decay_p1[h]));
       bs[t] = delta ? 1.f / (1.f + expf(-beta[n * beta_stride + beta_col + h])) : 1.f;
     }
+    }
     __syncthreads();
-    // a wave per token: unit norms (the rows scaled where they lie) and k . q, which the read-out needs
-    for (int t = wave; t < nt; t += n_waves) {
-      float* qrow = qs + t * DP;
-      float* krow = ks + t * DP;
+    // eight lanes a token: unit norms (the rows scaled where they lie) and k . q, which the read-out needs;
+    // the sums over a token's eight lanes are register exchanges
+    for (int t = threadIdx.x / 8; t < nt; t += blockDim.x / 8) {
+      const int s8 = threadIdx.x % 8;
+      float* qrow = qs + t * DS;
+      float* krow = ks + t * DS;
       float ssq = 0.f, ssk = 0.f, dot = 0.f;
-      for (int c = lane; c < DP; c += kWave) {
-        const float a = qrow[c], b = krow[c];
-        ssq = fmaf(a, a, ssq);
-        ssk = fmaf(b, b, ssk);
-        dot = fmaf(a, b, dot);
+      for (int c = 4 * s8; c < DP; c += 32) {
+        const float4 a = *reinterpret_cast<const float4*>(qrow + c), b = *reinterpret_cast<const float4*>(krow + c);
+        ssq = fmaf(a.x, a.x, fmaf(a.y, a.y, fmaf(a.z, a.z, fmaf(a.w, a.w, ssq))));
+        ssk = fmaf(b.x, b.x, fmaf(b.y, b.y, fmaf(b.z, b.z, fmaf(b.w, b.w, ssk))));
+        dot = fmaf(a.x, b.x, fmaf(a.y, b.y, fmaf(a.z, b.z, fmaf(a.w, b.w, dot))));
       }
-      dot = wave_sum(dot);
+      dot = column_sum<8>(dot);
       if (unit_eps >= 0.f) {
-        const float mq = q_scale / sqrtf(wave_sum(ssq) + unit_eps), mk = 1.f / sqrtf(wave_sum(ssk) + unit_eps);
-        for (int c = lane; c < DP; c += kWave) {
-          qrow[c] *= mq;
-          krow[c] *= mk;
+        const float mq = q_scale / sqrtf(column_sum<8>(ssq) + unit_eps), mk = 1.f / sqrtf(column_sum<8>(ssk) + unit_eps);
+        for (int c = 4 * s8; c < DP; c += 32) {
+          float4 a = *reinterpret_cast<const float4*>(qrow + c), b = *reinterpret_cast<const float4*>(krow + c);
+          a.x *= mq; a.y *= mq; a.z *= mq; a.w *= mq;
+          b.x *= mk; b.y *= mk; b.z *= mk; b.w *= mk;
+          *reinterpret_cast<float4*>(qrow + c) = a;
+          *reinterpret_cast<float4*>(krow + c) = b;
         }
         dot *= mq * mk;
       }
-      if (lane == 0) kqs[t] = dot;
+      if (s8 == 0) kqs[t] = dot;
     }
     __syncthreads();
-#pragma unroll 2
-    for (int t = 0; t < nt; ++t) {
-      const float4* kt = reinterpret_cast<const float4*>(ks + t * DP + sub * kScanRows);
-      const float4* qt = reinterpret_cast<const float4*>(qs + t * DP + sub * kScanRows);
-      float kr[kScanRows];
+    // the walk; a token's k, q and decays are read from LDS while the token before is worked on
+    float kn[kScanRows], qn[kScanRows], an[kScanRows];
+    auto fetch = [&](int t) {
+      const float4* kt = reinterpret_cast<const float4*>(ks + t * DS + sub * kScanRows);
+      const float4* qt = reinterpret_cast<const float4*>(qs + t * DS + sub * kScanRows);
 #pragma unroll
       for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
-        const float4 k4 = kt[r4];
-        kr[4 * r4] = k4.x; kr[4 * r4 + 1] = k4.y; kr[4 * r4 + 2] = k4.z; kr[4 * r4 + 3] = k4.w;
+        const float4 k4 = kt[r4], q4 = qt[r4];
+        kn[4 * r4] = k4.x; kn[4 * r4 + 1] = k4.y; kn[4 * r4 + 2] = k4.z; kn[4 * r4 + 3] = k4.w;
+        qn[4 * r4] = q4.x; qn[4 * r4 + 1] = q4.y; qn[4 * r4 + 2] = q4.z; qn[4 * r4 + 3] = q4.w;
       }
       if (decay_mode == 1) {
-        const float4* at = reinterpret_cast<const float4*>(as + t * DP + sub * kScanRows);
+        const float4* at = reinterpret_cast<const float4*>(as + t * DS + sub * kScanRows);
 #pragma unroll
         for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
           const float4 a4 = at[r4];
-          S[4 * r4] *= a4.x; S[4 * r4 + 1] *= a4.y; S[4 * r4 + 2] *= a4.z; S[4 * r4 + 3] *= a4.w;
+          an[4 * r4] = a4.x; an[4 * r4 + 1] = a4.y; an[4 * r4 + 2] = a4.z; an[4 * r4 + 3] = a4.w;
         }
+      }
+    };
+    fetch(0);
+#pragma unroll 2
+    for (int t = 0; t < nt; ++t) {
+      float kr[kScanRows], qr[kScanRows];
+#pragma unroll
+      for (int r = 0; r < kScanRows; ++r) {
+        kr[r] = kn[r];
+        qr[r] = qn[r];
+      }
+      if (decay_mode == 1) {
+#pragma unroll
+        for (int r = 0; r < kScanRows; ++r) S[r] *= an[r];
       } else {
         const float a = as[t];
 #pragma unroll
         for (int r = 0; r < kScanRows; ++r) S[r] *= a;
       }
+      const float v_t = vs[t * cols_per_block + col_local], b_t = bs[t], kq_t = kqs[t];
+      if (t + 1 < nt) fetch(t + 1);
       // both sums over the decayed S at once: S^T k for the write, S^T q for the read-out, which sees the
       // token's own write through q . (k u^T) = u (k . q)
       float pk[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
-      float qr[kScanRows];
-#pragma unroll
-      for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
-        const float4 q4 = qt[r4];
-        qr[4 * r4] = q4.x; qr[4 * r4 + 1] = q4.y; qr[4 * r4 + 2] = q4.z; qr[4 * r4 + 3] = q4.w;
-      }
 #pragma unroll
       for (int r = 0; r < kScanRows; ++r) {
         pk[r % 4] = fmaf(S[r], kr[r], pk[r % 4]);
         pq[r % 4] = fmaf(S[r], qr[r], pq[r % 4]);
       }
       const float sq = column_sum<TPC>((pq[0] + pq[1]) + (pq[2] + pq[3]));
-      float u = vs[t * cols_per_block + col_local];
-      if (delta) u = bs[t] * (u - column_sum<TPC>((pk[0] + pk[1]) + (pk[2] + pk[3])));
-      const float so = fmaf(u, kqs[t], sq);
+      float u = v_t;
+      if (delta) u = b_t * (u - column_sum<TPC>((pk[0] + pk[1]) + (pk[2] + pk[3])));
+      const float so = fmaf(u, kq_t, sq);
 #pragma unroll
       for (int r = 0; r < kScanRows; ++r) S[r] = fmaf(kr[r], u, S[r]);
       if (has_col && sub == 0) out[(static_cast<size_t>(q0 + t0 + t) * n_heads + h) * vdim + col] = so;
@@ -248,24 +383,30 @@ extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, 
   YK_REQUIRE(decay_mode == 0 || decay_mode == 1, "linear_state_scan: unknown kind of decay");
   YK_REQUIRE(decay != nullptr && decay_p0 != nullptr && (decay_mode == 1 || decay_p1 != nullptr), "linear_state_scan: the decay's inputs are missing");
   YK_REQUIRE(decay_mode == 0 || tau > 0.f, "linear_state_scan: tau must be positive");
-  YK_REQUIRE(dim <= kScanRows * kWave, "linear_state_scan: heads of more than 1,024 key channels are not offered");
+  YK_REQUIRE(dim <= kScanRowsMax * kWave, "linear_state_scan: heads of more than 1,024 key channels are not offered");
   if (n_seqs == 0) return 0;
+  // eight rows a lane while that leaves a column inside a wave (a wave's instructions per token are what
+  // the walk costs: fewer rows a lane, more lanes a column), sixteen beyond
+  const int rows = dim <= 8 * kWave ? 8 : 16;
   int tpc = 1;
-  while (tpc * kScanRows < dim) tpc *= 2;
-  int threads = vdim * tpc;
-  threads = std::min(256, (threads + kWave - 1) / kWave * kWave);
-  // (a decay per channel stages three padded rows a token: fewer threads where LDS would not hold more columns)
+  while (tpc * rows < dim) tpc *= 2;
+  // (always 256 threads: columns a workgroup has no use for idle in the walk but help to stage)
+  const int threads = 256;
   const int cols = threads / tpc;
   dim3 grid(n_seqs, n_heads, (vdim + cols - 1) / cols);
-  const size_t dp = static_cast<size_t>(tpc) * kScanRows;
+  const size_t dp = static_cast<size_t>(tpc) * rows;
   int chunk = kScanTokens;
-  const size_t per_token = sizeof(float) * (2 * dp + (decay_mode == 1 ? dp : 1) + cols + 2);
-  while (chunk > 4 && chunk * per_token > 100 * 1024) chunk /= 2;
+  const size_t per_token = sizeof(float) * (2 * (dp + 4) + (decay_mode == 1 ? dp + 4 : 1) + cols + 2);
+  while (chunk > 4 && (chunk * per_token > 110 * 1024 || chunk * dp > 8192)) chunk /= 2;
   const size_t lds = chunk * per_token;
   YK_REQUIRE(lds <= 128 * 1024, "linear_state_scan: the staged tokens do not fit in LDS");
+  auto al16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = dim % 8 == 0 && qkv_stride % 8 == 0 && (n_kv * dim) % 8 == 0 && al16(qkv) && chunk * dp <= 8192 &&
+                   (decay_mode == 0 || (decay_stride % 4 == 0 && decay_col % 4 == 0 && al16(decay) && al16(decay_p0)));
 #define YK_LAUNCH(T, TPC)                                                                                                       \
   {                                                                                                                             \
-    auto kern = linear_state_scan_kernel<T, TPC>;                                                                               \
+    auto kern = rows == 8 ? (vec ? linear_state_scan_kernel<T, TPC, 8, true> : linear_state_scan_kernel<T, TPC, 8, false>)      \
+                          : (vec ? linear_state_scan_kernel<T, TPC, 16, true> : linear_state_scan_kernel<T, TPC, 16, false>);   \
     if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                                static_cast<int>(lds)) != hipSuccess)                                            \
       return yk_fail("linear_state_scan: the staged tokens do not fit in LDS");                                                 \
