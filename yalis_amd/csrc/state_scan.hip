@@ -374,7 +374,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
 // and k are taken as they are.
 extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, int n_heads, int n_kv, int dim, int vdim,
                                     float* state, const int32_t* seq_qstart, const int32_t* seq_qlen,
-                                    const int32_t* state_slots, int n_seqs, float q_scale, float unit_eps, int decay_mode,
+                                    const int32_t* state_slots, int n_seqs, int n_tokens, float q_scale, float unit_eps, int decay_mode,
                                     const float* decay, int decay_stride, int decay_col, const float* decay_p0,
                                     const float* decay_p1, float tau, const float* beta, int beta_stride, int beta_col,
                                     float* out, hipStream_t stream) {
@@ -387,7 +387,9 @@ extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, 
   if (n_seqs == 0) return 0;
   // eight rows a lane while that leaves a column inside a wave (a wave's instructions per token are what
   // the walk costs: fewer rows a lane, more lanes a column), sixteen beyond
-  const int rows = dim <= 8 * kWave ? 8 : 16;
+  // (steps of single tokens are all staging and no walk: there the fewer, larger workgroups of sixteen rows
+  // a lane stage less twice)
+  const int rows = dim <= 8 * kWave && n_tokens > 4 * n_seqs ? 8 : 16;
   int tpc = 1;
   while (tpc * rows < dim) tpc *= 2;
   // (always 256 threads: columns a workgroup has no use for idle in the walk but help to stage)

@@ -114,7 +114,7 @@ _SIGNATURES = {
     "yk_latent_tile_tokens": ([_c_int], _c_int),
     "yk_latent_attention": ([_vp, _vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp], _c_int),
     "yk_linear_state_scan": (
-        [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_float, _c_float, _c_int, _vp, _c_int,
+        [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_int, _vp, _c_int,
          _c_int, _vp, _vp, _c_float, _vp, _c_int, _c_int, _vp, _vp],
         _c_int,
     ),
@@ -1524,7 +1524,7 @@ class HipOps:
         out = torch.empty((n, n_heads * vdim), dtype=torch.float32, device=qkv.device)
         self._check(self.lib.yk_linear_state_scan(
             qkv.data_ptr(), qkv.stride(0), _code(qkv.dtype), n_heads, n_kv, dim, vdim, state.data_ptr(), a["seq_qstart"].data_ptr(),
-            a["seq_qlen"].data_ptr(), a["state_slots"].data_ptr(), a["seq_qstart"].numel(), float(q_scale),
+            a["seq_qlen"].data_ptr(), a["state_slots"].data_ptr(), a["seq_qstart"].numel(), n, float(q_scale),
             -1.0 if unit_eps is None else float(unit_eps), 0 if kind == "head" else 1, src.data_ptr(), src.stride(0), col,
             p0.data_ptr(), _ptr(p1), tau, None if beta is None else beta[0].data_ptr(), 0 if beta is None else beta[0].stride(0),
             0 if beta is None else int(beta[1]), out.data_ptr(), self._stream()))
