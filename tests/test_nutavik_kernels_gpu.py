@@ -198,7 +198,8 @@ def test_one_row_stands_out_at_every_border(dtype, heads, kv_rank, rot_dim, spec
 @pytest.mark.parametrize("heads,in_dim,out_dim,tail,n", [(3, 32, 48, 8, 40), (16, 128, 512, 64, 150), (5, 512, 128, 0, 77), (2, 64, 16, 16, 33)])
 def test_head_linear_on_matrix_cores(heads, in_dim, out_dim, tail, n):
     """Many tokens, bfloat16 weights kept transposed: into the latent (bfloat16 in, a turned tail, float32
-    out) and out of it (float32 in, rounded as it is loaded, gates, bfloat16 out); token tiles that end
+    out) and out of it (float32 in as two bfloat16 parts, gates, bfloat16 out; also float32 out of the same
+    input to see that nothing of it was rounded away); token tiles that end
     inside a wave's 16 rows, column tiles that end inside a workgroup's 64."""
     o = ops()
     g = torch.Generator().manual_seed(n)
@@ -213,11 +214,14 @@ def test_head_linear_on_matrix_cores(heads, in_dim, out_dim, tail, n):
     got = o.head_linear(x.cuda(), w.cuda(), heads, in_dim, out_dim, torch.float32, tail=tail, rotation=on_device(rot) if tail else None,
                         positions=pos.cuda(), w_t=w_t)
     close(got, want, torch.float32, "into the latent", f32=2e-5)
-    xo = torch.randn(n, heads * in_dim, generator=g).to(bf).float()  # (values bfloat16 holds: the rounding at the load is exact)
+    xo = torch.randn(n, heads * in_dim, generator=g)  # (float32 values bfloat16 does not hold: they go in as two parts)
     gate = torch.randn(n, heads + 11, generator=g).to(bf)
     want = R.head_linear(xo, w, heads, in_dim, out_dim, bf, gate=gate, gate_col=7)
     got = o.head_linear(xo.cuda(), w.cuda(), heads, in_dim, out_dim, bf, gate=gate.cuda(), gate_col=7, w_t=w_t)
     close(got, want, bf, "out of the latent", bf16=1e-2)
+    # the same sums before their rounding: against the plain float32 product they differ by 2^-16 of the input, not 2^-8
+    exact = R.head_linear(xo, w, heads, in_dim, out_dim, torch.float32, gate=gate, gate_col=7)
+    assert (got.float().cpu() - exact.to(bf).float()).abs().max() <= 2.0 ** -7 * exact.abs().max()
 
 
 @pytest.mark.parametrize("heads,kv_rank,rot_dim,page", [(2, 64, 32, 32), (5, 128, 32, 64), (16, 512, 64, 64), (20, 256, 64, 32)])

@@ -208,8 +208,8 @@ extern "C" int yk_head_linear(const void* x, int x_stride, int x_dtype, const vo
 }
 
 // The same products on the matrix cores, for many tokens: bfloat16 weights kept [heads][out][in] (a row of
-// the second operand is then 16 bytes of memory a lane), the input bfloat16 or float32 (rounded as it is
-// loaded).  A wave makes 16 tokens x 64 columns of one head: the first operand is 16 input rows x 32
+// the second operand is then 16 bytes of memory a lane), the input bfloat16 or float32 (as two bfloat16
+// parts, the rounded value and what the rounding left over, each with its own product).  A wave makes 16 tokens x 64 columns of one head: the first operand is 16 input rows x 32
 // elements, loaded as it lies there.  Four waves a workgroup take four token tiles.
 typedef __bf16 hl_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float hl_f32x4_t __attribute__((ext_vector_type(4)));
@@ -229,6 +229,22 @@ template <>
 __device__ __forceinline__ hl_u32x4_t hl_load8<float>(const float* p) {
   const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
   return hl_u32x4_t{pack_bf16x2(a.x, a.y), pack_bf16x2(a.z, a.w), pack_bf16x2(b.x, b.y), pack_bf16x2(b.z, b.w)};
+}
+// what the rounding of eight floats to bfloat16 left over, itself rounded to bfloat16: a float32 input goes
+// through the matrix cores as the sum of the two, so the product sees it to 16 bits of fraction
+template <typename TX>
+__device__ __forceinline__ hl_u32x4_t hl_rest8(const TX* p, hl_u32x4_t hi);
+template <>
+__device__ __forceinline__ hl_u32x4_t hl_rest8<bf16_t>(const bf16_t*, hl_u32x4_t) {
+  return hl_u32x4_t{0u, 0u, 0u, 0u};
+}
+__device__ __forceinline__ uint32_t hl_rest2(float x, float y, uint32_t hi) {
+  return pack_bf16x2(x - __uint_as_float(hi << 16), y - __uint_as_float(hi & 0xffff0000u));
+}
+template <>
+__device__ __forceinline__ hl_u32x4_t hl_rest8<float>(const float* p, hl_u32x4_t hi) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  return hl_u32x4_t{hl_rest2(a.x, a.y, hi[0]), hl_rest2(a.z, a.w, hi[1]), hl_rest2(b.x, b.y, hi[2]), hl_rest2(b.z, b.w, hi[3])};
 }
 
 template <typename TX, typename TG, typename TO>
@@ -250,14 +266,16 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
   for (int j = 0; j < 4; ++j) acc[j] = hl_f32x4_t{0.f, 0.f, 0.f, 0.f};
   const int n_tiles = min(4, (out_dim - o0) / 16);
   for (int k0 = 0; k0 < in_dim; k0 += 32) {
-    HlFrag a;
+    HlFrag a, a_rest;
     a.u = hl_load8<TX>(xp + k0);
+    a_rest.u = hl_rest8<TX>(xp + k0, a.u);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (j < n_tiles) {
         HlFrag b;
         b.u = *reinterpret_cast<const hl_u32x4_t*>(wp + static_cast<size_t>(16 * j) * in_dim + k0);
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[j], 0, 0, 0);
+        if (sizeof(TX) == 4) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_rest.v, b.v, acc[j], 0, 0, 0);
       }
     }
   }

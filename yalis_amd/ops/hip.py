@@ -1397,7 +1397,7 @@ class HipOps:
         (float32 sums).  ``tail`` further elements of every head of x follow the product in the output,
         turned by the token's position (``rotation``, ``positions``); ``gate`` [N, >= gate_col + heads]:
         head h's output is multiplied by sigmoid(gate[n, gate_col + h]).  ``w_t`` (``head_weights_transposed``):
-        with it, products of many tokens run on the matrix cores (the input rounded to bfloat16 there)."""
+        with it, products of many tokens run on the matrix cores (a float32 input as two bfloat16 parts)."""
         self._rows(x, "head_linear input")
         n = x.shape[0]
         if tuple(w.shape) != (n_heads, in_dim, out_dim) or not w.is_contiguous() or x.shape[1] != n_heads * (in_dim + tail):
